@@ -1,0 +1,137 @@
+/*
+ * mercury_hip.h -- C ABI of the MI355X (gfx950) ring-attention step library.
+ *
+ * One shared library, libmercury_hip.so, plain pointers and sizes only.  Every pointer
+ * is a DEVICE pointer unless stated otherwise; `stream` is a hipStream_t passed as
+ * void* (NULL = the default stream).  All calls are asynchronous on `stream`, keep no
+ * global mutable state and allocate nothing.  Return value: 0 on success, a negative
+ * MHIP_E* code otherwise (mhip_error_string() gives the text).  Nothing throws.
+ *
+ * Tensor layouts follow the call sites of the reference (paths relative to the
+ * reference tree):
+ *   q, out, dout, dq      (B, Sq, Hq,  D)   element strides (sb, ss, sh), D contiguous
+ *   k, v, dk, dv          (B, Sc, Hkv, D)   element strides (sb, ss, sh), D contiguous
+ *   lse (block / final)   (B, Hq, Sq)  fp32 contiguous
+ *   merge accumulators    out (B, Sq, Hq, D) fp32, lse (B, Sq, Hq, 1) fp32, row strides given
+ *   packed reduce buffer  (B, Sq, Hq, D+1) fp32, out in [0,D), lse in column D
+ */
+#ifndef MERCURY_HIP_H_
+#define MERCURY_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- error codes --------------------------------------------------------------- */
+#define MHIP_OK              0
+#define MHIP_EINVAL         -1   /* bad size / NULL pointer / bad scale                 */
+#define MHIP_EDTYPE         -2   /* dtype code not supported by this entry point       */
+#define MHIP_EHEADDIM       -3   /* head dimension not supported (128 only)            */
+#define MHIP_EALIGN         -4   /* pointer or stride not 16-byte aligned              */
+#define MHIP_ELAUNCH        -5   /* hipLaunchKernel / hipGetLastError reported failure */
+#define MHIP_EUNSUPPORTED   -6   /* feature not implemented (dropout, alibi, window..) */
+
+/* ---- element types -------------------------------------------------------------- */
+#define MHIP_BF16  0
+#define MHIP_E4M3  1   /* OCP float8 e4m3fn */
+
+/* ---- mask classes of one (Q shard, KV chunk) block -------------------------------- */
+#define MHIP_MASK_NONE    0
+#define MHIP_MASK_CAUSAL  1   /* query i sees key j iff j <= i + (Sc - Sq) (bottom-right) */
+
+int         mhip_version(void);
+const char* mhip_error_string(int code);
+
+/*
+ * Block forward: out = softmax(scale * q k^T) v,  lse = logsumexp(scale * q k^T).
+ * Replaces flash_attn.flash_attn_interface._flash_attn_forward as called at
+ * utils/flash_attn_dsl.py:159-176 (dropout_p = 0, softcap = 0, no alibi, window (-1,-1)).
+ * out has q's element type for MHIP_BF16 and is bf16 for MHIP_E4M3.  Rows that see no key
+ * get out = 0 and lse = -inf.  For MHIP_E4M3 the three descales are the per-tensor fp32
+ * scales s (x ~ s * x_q); ignored for MHIP_BF16.
+ */
+int mhip_attn_fwd_block(const void* q, const void* k, const void* v, void* out, float* lse,
+                        int B, int Sq, int Sc, int Hq, int Hkv, int D,
+                        int64_t q_sb, int64_t q_ss, int64_t q_sh,
+                        int64_t k_sb, int64_t k_ss, int64_t k_sh,
+                        int64_t v_sb, int64_t v_ss, int64_t v_sh,
+                        int64_t o_sb, int64_t o_ss, int64_t o_sh,
+                        float softmax_scale, int mask, int dtype,
+                        float q_descale, float k_descale, float v_descale,
+                        void* stream);
+
+/*
+ * Block backward from the saved (final, merged) out and lse.
+ * Replaces flash_attn.flash_attn_interface._flash_attn_backward as called at
+ * utils/attn_bwd_dsl.py:83-115: writes every element of dq (B,Sq,Hq,D), dk and dv
+ * (B,Sc,Hkv,D) in bf16.  If dq_acc (fp32, contiguous (B,Sq,Hq,D)) is not NULL the block's
+ * dq is ALSO added into it in fp32 -- the `reduce(op=torch.add, buffer=reduce_dq, ...)`
+ * of utils/attn_bwd_dsl.py:117-122 folded into the kernel.  `workspace` must hold
+ * mhip_attn_bwd_workspace_bytes(...) bytes of device memory.
+ */
+int64_t mhip_attn_bwd_workspace_bytes(int B, int Sq, int Sc, int Hq, int Hkv, int D);
+int mhip_attn_bwd_block(const void* dout, const void* q, const void* k, const void* v,
+                        const void* out, const float* lse,
+                        void* dq, void* dk, void* dv, float* dq_acc,
+                        int B, int Sq, int Sc, int Hq, int Hkv, int D,
+                        int64_t q_sb, int64_t q_ss, int64_t q_sh,     /* q, out, dout, dq */
+                        int64_t k_sb, int64_t k_ss, int64_t k_sh,     /* k, v            */
+                        int64_t dk_sb, int64_t dk_ss, int64_t dk_sh,  /* dk, dv          */
+                        float softmax_scale, int mask, int deterministic,
+                        void* workspace, void* stream);
+
+/*
+ * LSE-rescale merge.  Replaces the TorchScript `_update_out_and_lse`
+ * (utils/flash_attn_dsl.py:31-49):
+ *     out' = out - sigmoid(bl - lse) * (out - bo),   lse' = lse - logsigmoid(lse - bl)
+ * with bo = float(block_out), bl = block_lse read transposed from (B,Hq,Sq).
+ * acc_out/acc_lse are read, dst_out/dst_lse written; dst may alias acc (the `slice_`
+ * path of utils/flash_attn_dsl.py:63-68 passes views, hence the strides: element strides
+ * of the (B,Sq,Hq) row index; D is contiguous).  A -inf operand is the identity.
+ * acc_out == NULL means "first call" (utils/flash_attn_dsl.py:61-62): dst = (bo, bl).
+ * If final_out / final_lse are not NULL the epilogue of utils/flash_attn_dsl.py:178-179 is
+ * fused: final_out (B,Sq,Hq,D) bf16 contiguous = bf16(out'), final_lse (B,Hq,Sq) = lse'.
+ * block_lse rows are addressed as block_lse[b*bl_sb + h*bl_sh + s].
+ */
+int mhip_lse_merge(const float* acc_out, const float* acc_lse,
+                   const void* block_out, const float* block_lse,
+                   float* dst_out, float* dst_lse,
+                   void* final_out, float* final_lse,
+                   int B, int Sq, int Hq, int D,
+                   int64_t ao_sb, int64_t ao_ss, int64_t ao_sh,
+                   int64_t al_sb, int64_t al_ss, int64_t al_sh,
+                   int64_t bo_sb, int64_t bo_ss, int64_t bo_sh,
+                   int64_t bl_sb, int64_t bl_sh,
+                   int64_t do_sb, int64_t do_ss, int64_t do_sh,
+                   int64_t dl_sb, int64_t dl_ss, int64_t dl_sh,
+                   void* stream);
+
+/*
+ * Packed merge.  Replaces TorchScript `flash_reduce` (utils/flash_attn_dsl.py:293-305):
+ * lhs, rhs, dst are contiguous fp32 (rows, D+1), 16-byte aligned; dst must not overlap lhs
+ * or rhs (the reference's flash_reduce returns a new tensor as well).
+ */
+int mhip_flash_reduce(const float* lhs, const float* rhs, float* dst,
+                      int64_t rows, int D, void* stream);
+
+/*
+ * Pack a block result: dst (B,Sq,Hq,D+1) fp32 contiguous =
+ * cat([float(block_out), block_lse^T], -1)   (utils/flash_attn_dsl.py:396).
+ * If lhs is not NULL the pack is fused with the reduce: dst = flash_reduce(lhs, pack(block));
+ * dst must not overlap lhs.  block_out (B,Sq,Hq,D) bf16 and block_lse (B,Hq,Sq) contiguous.
+ */
+int mhip_pack_reduce(const float* lhs, const void* block_out, const float* block_lse,
+                     float* dst, int B, int Sq, int Hq, int D, void* stream);
+
+/*
+ * Gradient accumulation `torch.add(buf, block.to(float32))` (utils/attn_bwd_dsl.py:117-129):
+ * dst = (acc ? acc : 0) + float(block), n elements, block in bf16; dst may alias acc.
+ */
+int mhip_grad_accumulate(const float* acc, const void* block, float* dst, int64_t n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MERCURY_HIP_H_ */

@@ -1,0 +1,39 @@
+"""MI355X (gfx950) implementation of the per-rank compute step of Mercury's ring attention.
+
+Importing the package registers the two block operators and exposes, under the names Mercury's
+generated code resolves in its ``exec`` namespace, everything that code calls:
+``_flash_attn_forward``, ``_flash_attn_backward``, ``get_default_args``, ``update_out_and_lse``,
+``flash_reduce`` and the rank/mesh index helpers.  ``namespace()`` returns them as a dict.
+"""
+from __future__ import annotations
+
+from . import _native
+from .flash_attn_interface import (_flash_attn_backward, _flash_attn_forward, attn_bwd_block,
+                                   attn_fwd_block)
+from .merge import (_update_out_and_lse, flash_reduce, get_default_args, grad_accumulate, merge_into,
+                    pack_block, update_out_and_lse)
+from .ring import (flash_attn_backward, flash_attn_expose_reduce, flash_attn_pack_kv,
+                   flash_attn_pack_split_kv, fp8_pack_split_kv, gqa_pack_kv, quantize_e4m3,
+                   zigzag_causal_pack_kv)
+from .schedule import (LocalRing, double_ring_order, get_src_dst_ranks, n_dim_to_one_dim,
+                       one_dim_to_n_dim, ring_divide_order, shift_tuple_element, single_ring_order,
+                       zigzag_blocks, zigzag_step)
+
+__version__ = "0.1.0"
+
+
+def namespace() -> dict:
+    """Names to place in the dict generated ring code is ``exec``-ed in (the reference fills it with
+    ``from utils.flash_attn_dsl import *`` and ``from mercury.backend import *``)."""
+    return {
+        "_flash_attn_forward": _flash_attn_forward,
+        "_flash_attn_backward": _flash_attn_backward,
+        "get_default_args": get_default_args,
+        "update_out_and_lse": update_out_and_lse,
+        "_update_out_and_lse": _update_out_and_lse,
+        "flash_reduce": flash_reduce,
+        "one_dim_to_n_dim": one_dim_to_n_dim,
+        "n_dim_to_one_dim": n_dim_to_one_dim,
+        "shift_tuple_element": shift_tuple_element,
+        "get_src_dst_ranks": get_src_dst_ranks,
+    }

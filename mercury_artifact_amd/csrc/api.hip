@@ -1,0 +1,73 @@
+// C ABI entry points for the attention block kernels: argument validation and dispatch.
+// The entry points of the elementwise kernels sit next to their kernels in lse_merge.hip.
+#include "mhip_common.hpp"
+
+namespace mhip {
+int attn_fwd_bf16(const void* q, const void* k, const void* v, void* out, float* lse,
+                  int B, int Sq, int Sc, int Hq, int Hkv,
+                  const int64_t* strides, float scale, int mask, hipStream_t stream);
+int fill_empty_block(void* out, float* lse, int B, int Sq, int Hq, int D,
+                     int64_t o_sb, int64_t o_ss, int64_t o_sh, hipStream_t stream);
+}  // namespace mhip
+
+using namespace mhip;
+
+extern "C" int mhip_version(void) { return 1; }
+
+extern "C" const char* mhip_error_string(int code) {
+  switch (code) {
+    case MHIP_OK: return "ok";
+    case MHIP_EINVAL: return "invalid argument (size, NULL pointer or softmax scale)";
+    case MHIP_EDTYPE: return "element type not supported by this entry point";
+    case MHIP_EHEADDIM: return "head dimension not supported (this build handles D = 128)";
+    case MHIP_EALIGN: return "pointer or stride not aligned to 16 bytes";
+    case MHIP_ELAUNCH: return "kernel launch failed";
+    case MHIP_EUNSUPPORTED: return "feature not implemented";
+    default: return "unknown error code";
+  }
+}
+
+namespace {
+bool mult8(int64_t x) { return (x & 7) == 0; }
+}  // namespace
+
+extern "C" int mhip_attn_fwd_block(const void* q, const void* k, const void* v, void* out, float* lse,
+                                   int B, int Sq, int Sc, int Hq, int Hkv, int D,
+                                   int64_t q_sb, int64_t q_ss, int64_t q_sh,
+                                   int64_t k_sb, int64_t k_ss, int64_t k_sh,
+                                   int64_t v_sb, int64_t v_ss, int64_t v_sh,
+                                   int64_t o_sb, int64_t o_ss, int64_t o_sh,
+                                   float softmax_scale, int mask, int dtype,
+                                   float q_descale, float k_descale, float v_descale,
+                                   void* stream) {
+  (void)q_descale; (void)k_descale; (void)v_descale;
+  if (B < 0 || Sq < 0 || Sc < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return MHIP_EINVAL;
+  if (!(softmax_scale > 0.f) || !(softmax_scale < INFINITY)) return MHIP_EINVAL;
+  if (mask != MHIP_MASK_NONE && mask != MHIP_MASK_CAUSAL) return MHIP_EINVAL;
+  if (dtype != MHIP_BF16 && dtype != MHIP_E4M3) return MHIP_EDTYPE;
+  if (D != 128) return MHIP_EHEADDIM;
+  if (B == 0 || Sq == 0) return MHIP_OK;
+  if (!q || !out || !lse) return MHIP_EINVAL;
+  if (Sc > 0 && (!k || !v)) return MHIP_EINVAL;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == MHIP_E4M3) return MHIP_EUNSUPPORTED;
+  // 16-byte vector accesses on every row of q, k, v and out
+  if (!aligned16(q) || !aligned16(out) || (Sc > 0 && (!aligned16(k) || !aligned16(v)))) return MHIP_EALIGN;
+  if (!mult8(q_sb) || !mult8(q_ss) || !mult8(q_sh) || !mult8(k_sb) || !mult8(k_ss) || !mult8(k_sh) ||
+      !mult8(v_sb) || !mult8(v_ss) || !mult8(v_sh) || !mult8(o_sb) || !mult8(o_ss) || !mult8(o_sh))
+    return MHIP_EALIGN;
+  const int64_t strides[12] = {q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, v_sb, v_ss, v_sh, o_sb, o_ss, o_sh};
+  return attn_fwd_bf16(q, k, v, out, lse, B, Sq, Sc, Hq, Hkv, strides, softmax_scale, mask, st);
+}
+
+extern "C" int64_t mhip_attn_bwd_workspace_bytes(int B, int Sq, int Sc, int Hq, int Hkv, int D) {
+  (void)B; (void)Sq; (void)Sc; (void)Hq; (void)Hkv; (void)D;
+  return 0;
+}
+
+extern "C" int mhip_attn_bwd_block(const void*, const void*, const void*, const void*, const void*,
+                                   const float*, void*, void*, void*, float*, int, int, int, int, int, int,
+                                   int64_t, int64_t, int64_t, int64_t, int64_t, int64_t,
+                                   int64_t, int64_t, int64_t, float, int, int, void*, void*) {
+  return MHIP_EUNSUPPORTED;
+}

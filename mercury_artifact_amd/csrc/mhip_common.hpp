@@ -1,0 +1,65 @@
+// Shared device/host helpers for the gfx950 ring-attention step kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mercury_hip.h"
+
+namespace mhip {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
+typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2;
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// Two fp32 -> one dword of two bf16 (round to nearest even), low half = a.
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  f32x2 v = {a, b};
+  bf16x2 r = __builtin_convertvector(v, bf16x2);
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+
+// max / sum of x over the lane pair (l, l ^ 32).  v_permlane32_swap exchanges the upper half of
+// its first operand with the lower half of its second, so with both operands = x every lane ends
+// up holding {own value, partner's value} in the two results (in an order that depends on the
+// half) -- a symmetric combine needs no lane test.  The two results are taken out as ints first:
+// __builtin_bit_cast applied directly to r[1] reads r[0] with this compiler.
+__device__ __forceinline__ void pair_exchange(float x, float& a, float& b) {
+  const int xi = __float_as_int(x);
+  auto r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
+  const int r0 = r[0], r1 = r[1];
+  a = __int_as_float(r0);
+  b = __int_as_float(r1);
+}
+__device__ __forceinline__ float pair_max(float x) {
+  float a, b;
+  pair_exchange(x, a, b);
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float pair_sum(float x) {
+  float a, b;
+  pair_exchange(x, a, b);
+  return a + b;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int launch_status() {
+  return hipGetLastError() == hipSuccess ? MHIP_OK : MHIP_ELAUNCH;
+}
+
+}  // namespace mhip

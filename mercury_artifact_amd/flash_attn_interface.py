@@ -1,0 +1,192 @@
+"""Block forward / backward operators with the keyword surface Mercury's generated ring code calls.
+
+The reference imports ``_flash_attn_forward`` / ``_flash_attn_backward`` from the third-party
+``flash_attn.flash_attn_interface`` (utils/flash_attn_dsl.py:6, utils/attn_bwd_dsl.py:8) and
+calls them by keyword with a dict built by ``get_default_args`` (utils/flash_attn_dsl.py:14-29,
+159-176; utils/attn_bwd_dsl.py:86-115).  The two operators below are registered through
+``torch.library.custom_op`` -- so ``get_default_args`` finds the Python signature on
+``._init_fn`` exactly as it does for flash-attn >= 2.7 -- and forward to the gfx950 kernels behind
+the C ABI of include/mercury_hip.h.  Binding these names into the namespace the generated code is
+``exec``-ed in replaces flash-attn without touching the generated code.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _native as N
+
+__all__ = ["_flash_attn_forward", "_flash_attn_backward", "attn_fwd_block", "attn_bwd_block"]
+
+
+def _strides3(t: torch.Tensor):
+    return t.stride(0), t.stride(1), t.stride(2)
+
+
+def _check_block_inputs(q, k, v, dropout_p, window_size_left, window_size_right, softcap, alibi_slopes):
+    N.require_cuda(q, k, v)
+    if dropout_p not in (0, 0.0, None):
+        raise RuntimeError("dropout_p != 0 is not supported (the ring templates always pass 0)")
+    if softcap not in (0, 0.0, None):
+        raise RuntimeError("softcap != 0 is not supported")
+    if alibi_slopes is not None:
+        raise RuntimeError("alibi_slopes is not supported")
+    if (window_size_left not in (-1, None)) or (window_size_right not in (-1, 0, None)):
+        raise RuntimeError("sliding windows are not supported (window_size must be (-1, -1))")
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise RuntimeError("q, k, v must be (batch, seq, heads, head_dim)")
+    if q.stride(-1) != 1 or k.stride(-1) != 1 or v.stride(-1) != 1:
+        raise RuntimeError("q, k, v must have a contiguous last dimension")
+    if k.shape != v.shape or q.shape[0] != k.shape[0] or q.shape[3] != k.shape[3]:
+        raise RuntimeError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
+    if q.shape[2] % k.shape[2] != 0:
+        raise RuntimeError("number of query heads must be a multiple of the number of KV heads")
+
+
+def attn_fwd_block(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float,
+                   causal: bool = False, q_descale: Optional[torch.Tensor] = None,
+                   k_descale: Optional[torch.Tensor] = None, v_descale: Optional[torch.Tensor] = None,
+                   out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
+                   ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(Q shard, one KV chunk) -> (out (B,Sq,Hq,D), lse (B,Hq,Sq) fp32) through mhip_attn_fwd_block."""
+    _check_block_inputs(q, k, v, 0, -1, -1, 0.0, None)
+    N.require_cuda(out, lse, q_descale, k_descale, v_descale)
+    B, Sq, Hq, D = q.shape
+    _, Sc, Hkv, _ = k.shape
+    if q.dtype == torch.bfloat16:
+        dt, out_dtype = N.MHIP_BF16, torch.bfloat16
+    elif q.dtype == torch.float8_e4m3fn:
+        dt, out_dtype = N.MHIP_E4M3, torch.bfloat16
+    else:
+        raise RuntimeError(f"unsupported dtype {q.dtype}: the gfx950 kernels take bfloat16 or float8_e4m3fn")
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise RuntimeError("q, k, v must share one dtype")
+    if out is None:
+        out = torch.empty((B, Sq, Hq, D), dtype=out_dtype, device=q.device)
+    elif out.shape != (B, Sq, Hq, D) or out.dtype != out_dtype or out.stride(-1) != 1:
+        raise RuntimeError("out must be (B, Sq, Hq, D) bfloat16 with a contiguous last dimension")
+    if lse is None:
+        lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
+    elif lse.shape != (B, Hq, Sq) or lse.dtype != torch.float32 or not lse.is_contiguous():
+        raise RuntimeError("lse must be a contiguous float32 (B, Hq, Sq) tensor")
+    ds = [1.0 if t is None else float(t) for t in (q_descale, k_descale, v_descale)]
+    with torch.cuda.device(q.device):
+        code = N.lib().mhip_attn_fwd_block(
+            N.ptr(q), N.ptr(k), N.ptr(v), N.ptr(out), N.ptr(lse),
+            B, Sq, Sc, Hq, Hkv, D,
+            *_strides3(q), *_strides3(k), *_strides3(v), *_strides3(out),
+            float(softmax_scale), N.MASK_CAUSAL if causal else N.MASK_NONE, dt,
+            ds[0], ds[1], ds[2], N.stream_of(q))
+    N.check(code, "mhip_attn_fwd_block")
+    return out, lse
+
+
+@torch.library.custom_op("mercury_amd::_flash_attn_forward", mutates_args=(), device_types="cuda")
+def _flash_attn_forward(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    dropout_p: float,
+    softmax_scale: float,
+    causal: bool,
+    window_size_left: int,
+    window_size_right: int,
+    softcap: float,
+    alibi_slopes: Optional[torch.Tensor],
+    return_softmax: bool,
+    q_descale: Optional[torch.Tensor] = None,
+    k_descale: Optional[torch.Tensor] = None,
+    v_descale: Optional[torch.Tensor] = None,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Returns ``(out, softmax_lse, S_dmask, rng_state)``; the last two are empty placeholders
+    (no dropout), kept because the generated code asserts ``len(outputs) == 4``
+    (utils/flash_attn_dsl.py:175)."""
+    _check_block_inputs(q, k, v, dropout_p, window_size_left, window_size_right, softcap, alibi_slopes)
+    out, lse = attn_fwd_block(q, k, v, softmax_scale, bool(causal), q_descale, k_descale, v_descale)
+    empty = torch.empty((0,), dtype=q.dtype if q.dtype == torch.bfloat16 else torch.bfloat16, device=q.device)
+    rng = torch.empty((2,), dtype=torch.int64, device=q.device)
+    return out, lse, empty, rng
+
+
+@_flash_attn_forward.register_fake
+def _(q, k, v, dropout_p, softmax_scale, causal, window_size_left, window_size_right, softcap,
+      alibi_slopes, return_softmax, q_descale=None, k_descale=None, v_descale=None):
+    B, Sq, Hq, D = q.shape
+    od = torch.bfloat16
+    return (q.new_empty((B, Sq, Hq, D), dtype=od), q.new_empty((B, Hq, Sq), dtype=torch.float32),
+            q.new_empty((0,), dtype=od), q.new_empty((2,), dtype=torch.int64))
+
+
+def attn_bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_scale, causal=False,
+                   deterministic=False, dq_acc: Optional[torch.Tensor] = None) -> None:
+    """Block backward through mhip_attn_bwd_block; writes dq, dk, dv in place."""
+    B, Sq, Hq, D = q.shape
+    _, Sc, Hkv, _ = k.shape
+    for name, t in (("dout", dout), ("out", out), ("dq", dq)):
+        if t.shape != q.shape or t.stride() != q.stride():
+            if t.shape != q.shape:
+                raise RuntimeError(f"{name} must have q's shape")
+    lib = N.lib()
+    ws_bytes = lib.mhip_attn_bwd_workspace_bytes(B, Sq, Sc, Hq, Hkv, D)
+    ws = torch.empty((max(int(ws_bytes), 1),), dtype=torch.uint8, device=q.device)
+    doutc = dout if dout.stride() == q.stride() else dout.contiguous()
+    outc = out if out.stride() == q.stride() else out.contiguous()
+    qc = q
+    if doutc.stride() != qc.stride() or outc.stride() != qc.stride():
+        qc, doutc, outc = q.contiguous(), dout.contiguous(), out.contiguous()
+    dq_tmp = dq if dq.stride() == qc.stride() else torch.empty_like(qc)
+    if k.stride() != v.stride():
+        k, v = k.contiguous(), v.contiguous()
+    dk_tmp, dv_tmp = dk, dv
+    if dk.stride() != dv.stride():
+        dk_tmp, dv_tmp = torch.empty_like(dk, memory_format=torch.contiguous_format), \
+            torch.empty_like(dv, memory_format=torch.contiguous_format)
+    with torch.cuda.device(q.device):
+        code = lib.mhip_attn_bwd_block(
+            N.ptr(doutc), N.ptr(qc), N.ptr(k), N.ptr(v), N.ptr(outc), N.ptr(softmax_lse),
+            N.ptr(dq_tmp), N.ptr(dk_tmp), N.ptr(dv_tmp), N.ptr(dq_acc),
+            B, Sq, Sc, Hq, Hkv, D,
+            *_strides3(qc), *_strides3(k), *_strides3(dk_tmp),
+            float(softmax_scale), N.MASK_CAUSAL if causal else N.MASK_NONE, int(bool(deterministic)),
+            N.ptr(ws), N.stream_of(q))
+    N.check(code, "mhip_attn_bwd_block")
+    if dq_tmp is not dq:
+        dq.copy_(dq_tmp)
+    if dk_tmp is not dk:
+        dk.copy_(dk_tmp)
+        dv.copy_(dv_tmp)
+
+
+@torch.library.custom_op("mercury_amd::_flash_attn_backward", mutates_args=("dq", "dk", "dv"),
+                         device_types="cuda")
+def _flash_attn_backward(
+    dout: torch.Tensor,
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    out: torch.Tensor,
+    softmax_lse: torch.Tensor,
+    dq: torch.Tensor,
+    dk: torch.Tensor,
+    dv: torch.Tensor,
+    dropout_p: float,
+    softmax_scale: float,
+    causal: bool,
+    window_size_left: int,
+    window_size_right: int,
+    softcap: float,
+    alibi_slopes: Optional[torch.Tensor],
+    deterministic: bool,
+    rng_state: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Keyword surface of utils/attn_bwd_dsl.py:86-115; dq/dk/dv are caller-allocated
+    (``torch.empty``, utils/attn_bwd_dsl.py:83-84) and every element of them is written.
+    Returns ``softmax_d`` (rowsum(dout * out), (B,Hq,Sq) fp32) like flash-attn does."""
+    _check_block_inputs(q, k, v, dropout_p, window_size_left, window_size_right, softcap, alibi_slopes)
+    N.require_cuda(dout, out, softmax_lse, dq, dk, dv)
+    if q.dtype != torch.bfloat16:
+        raise RuntimeError("the backward kernel takes bfloat16 only")
+    attn_bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_scale, bool(causal),
+                   bool(deterministic))
+    return (dout.float() * out.float()).sum(-1).transpose(1, 2).contiguous()

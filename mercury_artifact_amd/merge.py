@@ -1,0 +1,162 @@
+"""Merge helpers the generated ring code calls by bare name.
+
+Same names, arguments and error behaviour as utils/flash_attn_dsl.py:14-71, 293-305 of the
+reference; the arithmetic runs in the gfx950 kernels behind mhip_lse_merge / mhip_flash_reduce /
+mhip_pack_reduce.  GPU tensors only.
+"""
+from __future__ import annotations
+
+import inspect
+from functools import cache
+from typing import Optional, Tuple
+
+import torch
+
+from . import _native as N
+
+__all__ = ["get_default_args", "update_out_and_lse", "_update_out_and_lse", "flash_reduce",
+           "pack_block", "merge_into", "grad_accumulate"]
+
+
+@cache
+def _get_default_args(func):
+    spec = inspect.getfullargspec(func)
+    defaults = spec.defaults if spec.defaults is not None else ()
+    padded = (None,) * (len(spec.args) - len(defaults)) + tuple(defaults)
+    args = dict(zip(spec.args, padded))
+    if "softcap" in args:
+        args["softcap"] = 0.0
+    return args
+
+
+def get_default_args(func):
+    """utils/flash_attn_dsl.py:24-29: keyword -> default of ``func`` (or of the Python function
+    a ``torch.library`` custom op was created from), parameters without a default mapped to
+    ``None`` and ``softcap`` forced to 0.0.  The caller copies the dict before updating it."""
+    if inspect.isfunction(func):
+        return _get_default_args(func)
+    return _get_default_args(func._init_fn)
+
+
+def _row_strides(t: torch.Tensor):
+    return t.stride(0), t.stride(1), t.stride(2)
+
+
+def merge_into(acc_out: Optional[torch.Tensor], acc_lse: Optional[torch.Tensor],
+               block_out: torch.Tensor, block_lse: torch.Tensor,
+               dst_out: Optional[torch.Tensor], dst_lse: Optional[torch.Tensor],
+               final_out: Optional[torch.Tensor] = None, final_lse: Optional[torch.Tensor] = None) -> None:
+    """One call of mhip_lse_merge.  acc (B,Sq,Hq,D)/(B,Sq,Hq,1) fp32 or None for the first block,
+    block_out (B,Sq,Hq,D) bf16, block_lse (B,Hq,Sq) fp32, dst like acc (may be acc itself),
+    final_out (B,Sq,Hq,D) bf16 contiguous and final_lse (B,Hq,Sq) fp32 contiguous or None."""
+    N.require_cuda(acc_out, acc_lse, block_out, block_lse, dst_out, dst_lse, final_out, final_lse)
+    B, Sq, Hq, D = block_out.shape
+    if block_out.dtype != torch.bfloat16 or block_out.stride(-1) != 1:
+        raise RuntimeError("block_out must be bfloat16 with a contiguous last dimension")
+    if block_lse.shape != (B, Hq, Sq) or block_lse.dtype != torch.float32 or block_lse.stride(2) != 1:
+        raise RuntimeError("block_lse must be float32 (B, Hq, Sq) with contiguous rows")
+    for name, o, l in (("acc", acc_out, acc_lse), ("dst", dst_out, dst_lse)):
+        if o is None:
+            continue
+        if o.shape != (B, Sq, Hq, D) or l.shape != (B, Sq, Hq, 1):
+            raise RuntimeError(f"{name} shapes {tuple(o.shape)} / {tuple(l.shape)} do not match the block")
+        if o.dtype != torch.float32 or l.dtype != torch.float32 or o.stride(-1) != 1:
+            raise RuntimeError(f"{name} must be float32 with a contiguous last dimension")
+    if final_out is not None:
+        if not (final_out.is_contiguous() and final_lse.is_contiguous()):
+            raise RuntimeError("final_out / final_lse must be contiguous")
+        if final_out.shape != (B, Sq, Hq, D) or final_lse.shape != (B, Hq, Sq):
+            raise RuntimeError("final_out / final_lse shapes do not match the block")
+    z3 = (0, 0, 0)
+    with torch.cuda.device(block_out.device):
+        code = N.lib().mhip_lse_merge(
+            N.ptr(acc_out), N.ptr(acc_lse), N.ptr(block_out), N.ptr(block_lse),
+            N.ptr(dst_out), N.ptr(dst_lse), N.ptr(final_out), N.ptr(final_lse),
+            B, Sq, Hq, D,
+            *(z3 if acc_out is None else _row_strides(acc_out)),
+            *(z3 if acc_lse is None else _row_strides(acc_lse)),
+            *_row_strides(block_out), block_lse.stride(0), block_lse.stride(1),
+            *(z3 if dst_out is None else _row_strides(dst_out)),
+            *(z3 if dst_lse is None else _row_strides(dst_lse)),
+            N.stream_of(block_out))
+    N.check(code, "mhip_lse_merge")
+
+
+def _update_out_and_lse(out: torch.Tensor, lse: torch.Tensor, block_out: torch.Tensor,
+                        block_lse: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """utils/flash_attn_dsl.py:31-49 -- functional: returns new (out, lse), inputs untouched."""
+    block_out = block_out if block_out.dtype == torch.bfloat16 else block_out.to(torch.bfloat16)
+    new_out = torch.empty(out.shape, dtype=torch.float32, device=out.device)
+    new_lse = torch.empty(lse.shape, dtype=torch.float32, device=lse.device)
+    merge_into(out, lse, block_out, block_lse, new_out, new_lse)
+    return new_out, new_lse
+
+
+def update_out_and_lse(out: Optional[torch.Tensor], lse: Optional[torch.Tensor],
+                       block_out: torch.Tensor, block_lse: torch.Tensor, slice_=None,
+                       ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """utils/flash_attn_dsl.py:51-71.  First call (``out is None``) turns the block into the fp32
+    accumulators; ``slice_`` merges into that sub-range of the accumulators in place; otherwise a
+    functional merge."""
+    if out is None:
+        if slice_ is not None:
+            raise RuntimeError("first update_out_and_lse should not pass slice_ args")
+        B, Sq, Hq, D = block_out.shape
+        out = torch.empty((B, Sq, Hq, D), dtype=torch.float32, device=block_out.device)
+        lse = torch.empty((B, Sq, Hq, 1), dtype=torch.float32, device=block_out.device)
+        merge_into(None, None, block_out, block_lse, out, lse)
+    elif slice_ is not None:
+        so, sl = out[slice_], lse[slice_]
+        merge_into(so, sl, block_out, block_lse, so, sl)
+    else:
+        out, lse = _update_out_and_lse(out, lse, block_out, block_lse)
+    return out, lse
+
+
+def flash_reduce(lhs: torch.Tensor, rhs: torch.Tensor) -> torch.Tensor:
+    """utils/flash_attn_dsl.py:293-305 on packed ``[..., D+1]`` fp32 operands; returns a new tensor."""
+    N.require_cuda(lhs, rhs)
+    if lhs.shape != rhs.shape or lhs.dtype != torch.float32 or rhs.dtype != torch.float32:
+        raise RuntimeError("flash_reduce takes two float32 tensors of one shape")
+    lhs, rhs = lhs.contiguous(), rhs.contiguous()
+    dst = torch.empty_like(lhs)
+    W = lhs.shape[-1]
+    rows = lhs.numel() // W if W else 0
+    with torch.cuda.device(lhs.device):
+        code = N.lib().mhip_flash_reduce(N.ptr(lhs), N.ptr(rhs), N.ptr(dst), rows, W - 1, N.stream_of(lhs))
+    N.check(code, "mhip_flash_reduce")
+    return dst
+
+
+def pack_block(block_out: torch.Tensor, block_lse: torch.Tensor,
+               reduce_into: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``torch.cat([block_out.float(), block_lse.transpose(-2,-1).unsqueeze(-1)], -1)``
+    (utils/flash_attn_dsl.py:396) in one pass; with ``reduce_into`` the result is
+    ``flash_reduce(reduce_into, pack)`` without materialising the pack."""
+    N.require_cuda(block_out, block_lse, reduce_into)
+    B, Sq, Hq, D = block_out.shape
+    block_out, block_lse = block_out.contiguous(), block_lse.contiguous()
+    if block_out.dtype != torch.bfloat16:
+        raise RuntimeError("block_out must be bfloat16")
+    dst = torch.empty((B, Sq, Hq, D + 1), dtype=torch.float32, device=block_out.device)
+    lhs = None if reduce_into is None else reduce_into.contiguous()
+    with torch.cuda.device(block_out.device):
+        code = N.lib().mhip_pack_reduce(N.ptr(lhs), N.ptr(block_out), N.ptr(block_lse), N.ptr(dst),
+                                        B, Sq, Hq, D, N.stream_of(block_out))
+    N.check(code, "mhip_pack_reduce")
+    return dst
+
+
+def grad_accumulate(acc: Optional[torch.Tensor], block: torch.Tensor) -> torch.Tensor:
+    """``torch.add(acc, block.to(torch.float32))`` (utils/attn_bwd_dsl.py:117-129); ``acc is None``
+    is the first chunk (codegen.py:99-115 emits a plain assignment there)."""
+    N.require_cuda(acc, block)
+    if block.dtype != torch.bfloat16:
+        raise RuntimeError("block must be bfloat16")
+    block = block.contiguous()
+    dst = torch.empty(block.shape, dtype=torch.float32, device=block.device)
+    a = None if acc is None else acc.contiguous()
+    with torch.cuda.device(block.device):
+        code = N.lib().mhip_grad_accumulate(N.ptr(a), N.ptr(block), N.ptr(dst), block.numel(), N.stream_of(block))
+    N.check(code, "mhip_grad_accumulate")
+    return dst

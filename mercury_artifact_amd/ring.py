@@ -1,0 +1,256 @@
+"""Fixed-schedule drivers of one rank's ring-attention step on one GPU.
+
+Each driver has the argument list of the function Mercury generates from the template of the same
+name (utils/flash_attn_dsl.py:127-180, 182-235, 237-291, 345-408; utils/attn_bwd_dsl.py:37-135) plus a
+``ring`` keyword: the :class:`~mercury_artifact_amd.schedule.LocalRing` that stands in for the
+neighbour exchange.  The body is the loop the code generator emits for that template
+(mercury/backend/pytorch/codegen.py:264-355, 443-523): take the current KV chunk, start the hop for
+the next one, run the block kernel through ``_flash_attn_forward(**params)``, fold with
+``update_out_and_lse``, and store after the last step.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .flash_attn_interface import _flash_attn_backward, _flash_attn_forward
+from .merge import get_default_args, grad_accumulate, merge_into, pack_block, update_out_and_lse
+from .schedule import LocalRing, n_dim_to_one_dim, one_dim_to_n_dim, shift_tuple_element, zigzag_step
+
+__all__ = ["flash_attn_pack_kv", "gqa_pack_kv", "flash_attn_pack_split_kv", "flash_attn_expose_reduce",
+           "flash_attn_backward", "zigzag_causal_pack_kv", "fp8_pack_split_kv", "quantize_e4m3"]
+
+
+def _hops(ring: LocalRing):
+    """(dim, is_last) per step in generated-loop order: innermost mesh dimension first, a hop on
+    the next dimension when the inner loop wraps, nothing after the very last step."""
+    shape = ring.mesh_shape
+    total = ring.world
+    idx = [0] * len(shape)
+    for step in range(total):
+        hop = None
+        for d in range(len(shape)):
+            if idx[d] + 1 != shape[d]:
+                hop = d
+                break
+        yield hop
+        # advance the odometer (dimension 0 fastest)
+        for d in range(len(shape)):
+            idx[d] += 1
+            if idx[d] < shape[d]:
+                break
+            idx[d] = 0
+
+
+def _neighbours(ring: LocalRing, dim: int):
+    me = one_dim_to_n_dim(ring.rank, ring.mesh_shape)
+    size = ring.mesh_shape[dim]
+    send_to = n_dim_to_one_dim(shift_tuple_element(me, dim, 1, size), ring.mesh_shape)
+    recv_from = n_dim_to_one_dim(shift_tuple_element(me, dim, -1, size), ring.mesh_shape)
+    return send_to, recv_from
+
+
+def _fwd_params(q, k, v, softmax_scale, dropout_p, causal, window_size, alibi_slopes, **extra):
+    params = get_default_args(_flash_attn_forward).copy()
+    params.update({
+        "q": q, "k": k, "v": v,
+        "dropout_p": dropout_p,
+        "softmax_scale": softmax_scale,
+        "causal": causal,
+        "alibi_slopes": alibi_slopes,
+        "return_softmax": True and dropout_p > 0,
+        "window_size_left": window_size[0],
+        "window_size_right": window_size[1],
+    })
+    params.update(extra)
+    return params
+
+
+def _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes,
+                  ring: LocalRing, fused_epilogue: bool, **extra):
+    _out = None
+    _lse = None
+    _kv = None
+    _next_kv = None
+    steps = list(_hops(ring))
+    for step, hop in enumerate(steps):
+        if step == 0:
+            _kv = kv.contiguous()
+        else:
+            ring.wait()
+            _kv = _next_kv
+        if hop is not None:
+            send_to, recv_from = _neighbours(ring, hop)
+            _next_kv = ring.send_recv(send_to, recv_from, _kv)
+            ring.commit()
+        _k = _kv[0]
+        _v = _kv[1]
+        outputs = _flash_attn_forward(**_fwd_params(q, _k, _v, softmax_scale, dropout_p, causal,
+                                                    window_size, alibi_slopes, **extra))
+        assert len(outputs) == 4
+        block_out, block_lse, _, _ = outputs
+        if fused_epilogue and step + 1 == len(steps):
+            # last merge writes o / lse directly (same arithmetic, two passes fewer)
+            merge_into(_out, _lse, block_out, block_lse, None, None, o, lse)
+            return
+        _out, _lse = update_out_and_lse(_out, _lse, block_out, block_lse)
+    o[:, :, :, :] = _out.to(o.dtype)
+    lse[:, :, :] = _lse.squeeze(dim=-1).transpose(1, 2)
+
+
+def flash_attn_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False, window_size=(-1, -1),
+                       alibi_slopes=None, deterministic=False, *, ring: LocalRing,
+                       fused_epilogue: bool = False):
+    """Single-ring forward step (template utils/flash_attn_dsl.py:127-180).  q (B,Sq,H,D), kv the
+    rank's own (2,B,Sc,H,D), o (B,Sq,H,D) and lse (B,H,Sq) are written."""
+    _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes, ring,
+                  fused_epilogue)
+
+
+def gqa_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False, window_size=(-1, -1),
+                alibi_slopes=None, deterministic=False, *, ring: LocalRing, fused_epilogue: bool = False):
+    """GQA forward step (template utils/flash_attn_dsl.py:182-235): kv has Hkv heads, q has
+    Hkv * HEADS_PER_GROUP; the block kernel maps q head h to kv head h // HEADS_PER_GROUP."""
+    _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes, ring,
+                  fused_epilogue)
+
+
+def flash_attn_pack_split_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False,
+                             window_size=(-1, -1), alibi_slopes=None, deterministic=False, *,
+                             ring: LocalRing, fused_epilogue: bool = False):
+    """Double-ring forward step (template utils/flash_attn_dsl.py:237-291): ``ring`` is built on the
+    2-D mesh ``(inner, outer)``; the loop order and hops follow from the mesh shape."""
+    if len(ring.mesh_shape) != 2:
+        raise ValueError("the double ring needs a 2-D mesh (inner, outer)")
+    _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes, ring,
+                  fused_epilogue)
+
+
+def flash_attn_expose_reduce(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False,
+                             window_size=(-1, -1), alibi_slopes=None, deterministic=False, *,
+                             ring: LocalRing):
+    """Managed-reduction form (template utils/flash_attn_dsl.py:345-408) with the KV ring: block
+    results are packed ``(out | lse)`` and folded by ``flash_reduce``; pack and reduce run as one
+    kernel."""
+    buf = None
+    _kv = None
+    _next_kv = None
+    for step, hop in enumerate(_hops(ring)):
+        if step == 0:
+            _kv = kv.contiguous()
+        else:
+            ring.wait()
+            _kv = _next_kv
+        if hop is not None:
+            send_to, recv_from = _neighbours(ring, hop)
+            _next_kv = ring.send_recv(send_to, recv_from, _kv)
+            ring.commit()
+        outputs = _flash_attn_forward(**_fwd_params(q, _kv[0], _kv[1], softmax_scale, dropout_p, causal,
+                                                    window_size, alibi_slopes))
+        assert len(outputs) == 4
+        block_out, block_lse, _, _ = outputs
+        buf = pack_block(block_out, block_lse, reduce_into=buf)
+    o[:, :, :, :] = buf[..., :-1].to(o.dtype)
+    lse[:, :, :] = buf[..., -1].transpose(1, 2)
+
+
+def zigzag_causal_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=True, window_size=(-1, -1),
+                          alibi_slopes=None, deterministic=False, *, ring: LocalRing):
+    """Causal forward step in the zigzag layout (rank r holds sequence blocks r and 2W-1-r).  Not in
+    the reference, which only carries the ``slice_`` hook (utils/flash_attn_dsl.py:56,63-68); the
+    three step classes are the diagonal (causal block), "first half of the chunk" and "second half
+    of the Q rows" (merged through ``slice_``)."""
+    if len(ring.mesh_shape) != 1:
+        raise ValueError("zigzag runs on a 1-D ring")
+    world = ring.world
+    Sq = q.shape[1]
+    if Sq % 2 or kv.shape[2] != Sq:
+        raise ValueError("zigzag needs an even number of local rows and equal Q / KV shards")
+    half = Sq // 2
+    _out = _lse = _kv = _next_kv = None
+    for step in range(world):
+        if step == 0:
+            _kv = kv.contiguous()
+        else:
+            ring.wait()
+            _kv = _next_kv
+        if step + 1 != world:
+            send_to, recv_from = _neighbours(ring, 0)
+            _next_kv = ring.send_recv(send_to, recv_from, _kv)
+            ring.commit()
+        kind, _ = zigzag_step(ring.rank, step, world)
+        if kind == "diag":
+            bq, bk, bv, bc, sl = q, _kv[0], _kv[1], True, None
+        elif kind == "kv_first_half":
+            bq, bk, bv, bc, sl = q, _kv[0][:, :half], _kv[1][:, :half], False, None
+        else:
+            bq, bk, bv, bc, sl = q[:, half:], _kv[0], _kv[1], False, (slice(None), slice(half, None))
+        outputs = _flash_attn_forward(**_fwd_params(bq, bk, bv, softmax_scale, dropout_p, bc,
+                                                    window_size, alibi_slopes))
+        block_out, block_lse, _, _ = outputs
+        _out, _lse = update_out_and_lse(_out, _lse, block_out, block_lse, slice_=sl)
+    o[:, :, :, :] = _out.to(o.dtype)
+    lse[:, :, :] = _lse.squeeze(dim=-1).transpose(1, 2)
+
+
+def quantize_e4m3(x: torch.Tensor):
+    """Per-tensor e4m3 quantisation: scale s = amax / 448 (fp32), x_q = round-to-nearest-even(x / s)."""
+    amax = x.abs().amax().to(torch.float32)
+    scale = torch.where(amax > 0, amax / 448.0, torch.ones_like(amax))
+    xq = (x.to(torch.float32) / scale).clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
+    return xq, scale
+
+
+def fp8_pack_split_kv(q, kv, o, lse, softmax_scale, q_descale, k_descale, v_descale, dropout_p=0,
+                      causal=False, window_size=(-1, -1), alibi_slopes=None, deterministic=False, *,
+                      ring: LocalRing, fused_epilogue: bool = False):
+    """Forward step on e4m3 Q/K/V with per-tensor descales (not in the reference); any mesh."""
+    _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes, ring,
+                  fused_epilogue, q_descale=q_descale, k_descale=k_descale, v_descale=v_descale)
+
+
+def flash_attn_backward(q, kv, o, lse, dout, dq, dkv, softmax_scale, dropout_p=0, causal=False,
+                        window_size=(-1, -1), alibi_slopes=None, deterministic=False, *,
+                        ring: LocalRing, dkv_chunks: Optional[dict] = None):
+    """Backward ring step (template utils/attn_bwd_dsl.py:37-135 after ``shift`` on the KV axis):
+    KV chunks arrive in ring order, each gets a block backward against the local q / o / lse / dout;
+    dq accumulates in fp32 over the chunks (utils/attn_bwd_dsl.py:117-122) and is stored as
+    ``dq.dtype`` at the end (131-132).  The fp32 dK/dV accumulator that travels with its chunk on a
+    real ring has exactly one contribution per rank, so here each chunk's block gradient is kept in
+    ``dkv_chunks[chunk id]`` (fp32) and the rank's own chunk is stored to ``dkv``."""
+    reduce_dq = None
+    _kv = _next_kv = None
+    own = ring.current
+    for step, hop in enumerate(_hops(ring)):
+        if step == 0:
+            _kv = kv.contiguous()
+        else:
+            ring.wait()
+            _kv = _next_kv
+        chunk_id = ring.current
+        if hop is not None:
+            send_to, recv_from = _neighbours(ring, hop)
+            _next_kv = ring.send_recv(send_to, recv_from, _kv)
+            ring.commit()
+        block_dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        block_dkv = torch.empty(_kv.shape, dtype=kv.dtype, device=kv.device)
+        params = get_default_args(_flash_attn_backward).copy()
+        params.update({
+            "dout": dout, "q": q, "k": _kv[0], "v": _kv[1], "out": o, "softmax_lse": lse,
+            "dq": block_dq, "dk": block_dkv[0], "dv": block_dkv[1],
+            "softmax_scale": softmax_scale, "dropout_p": dropout_p, "causal": False,
+            "deterministic": deterministic, "alibi_slopes": alibi_slopes,
+        })
+        if "window_size" in params:
+            params.update({"window_size": window_size})
+        else:
+            params.update({"window_size_left": window_size[0], "window_size_right": window_size[1]})
+        _flash_attn_backward(**params)
+        reduce_dq = grad_accumulate(reduce_dq, block_dq)
+        red = grad_accumulate(None, block_dkv)
+        if dkv_chunks is not None:
+            dkv_chunks[chunk_id] = red
+        if chunk_id == own:
+            dkv[...] = red.to(dkv.dtype)
+    dq[...] = reduce_dq.to(dq.dtype)

@@ -1,0 +1,124 @@
+"""Merge kernels (through the C ABI) against the CPU oracle.
+
+fp32 elementwise arithmetic: the kernel evaluates the same sigmoid / softplus expressions with
+different intrinsics, so the tolerance is a few fp32 ulps of the operands: atol = rtol = 2e-6 on
+out and lse (the reference's own tests accept 1e-3)."""
+import math
+
+import pytest
+import torch
+
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = dict(atol=2e-6, rtol=2e-6)
+
+
+def _blocks(B, Sq, H, D, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    out = torch.randn(B, Sq, H, D, generator=g)
+    lse = torch.randn(B, Sq, H, 1, generator=g) * 3 + 5
+    bo = torch.randn(B, Sq, H, D, generator=g).bfloat16()
+    bl = torch.randn(B, H, Sq, generator=g) * 3 + 5
+    return out, lse, bo, bl
+
+
+@pytest.mark.parametrize("B,Sq,H,D", [(1, 64, 4, 128), (2, 37, 3, 128), (1, 5, 1, 128), (2, 33, 5, 64),
+                                      (1, 19, 2, 32), (1, 9, 2, 256), (1, 21, 3, 40)])
+def test_update_out_and_lse_matches_reference_formula(B, Sq, H, D):
+    import mercury_artifact_amd as M
+
+    print(f"merge case {B} {Sq} {H} {D}", flush=True)
+    out, lse, bo, bl = _blocks(B, Sq, H, D)
+    ro, rl = O.merge_reference(out, lse, bo, bl)
+    od, ld, bod, bld = out.cuda(), lse.cuda(), bo.cuda(), bl.cuda()
+    # first call
+    fo, fl = M.update_out_and_lse(None, None, bod, bld)
+    assert torch.equal(fo.cpu(), bo.float()) and torch.equal(fl.cpu()[..., 0], bl.transpose(1, 2))
+    # functional merge leaves its inputs alone
+    no, nl = M.update_out_and_lse(od, ld, bod, bld)
+    assert torch.equal(od.cpu(), out) and torch.equal(ld.cpu(), lse)
+    assert torch.allclose(no.cpu(), ro, **TOL) and torch.allclose(nl.cpu(), rl, **TOL)
+    # slice_ path merges in place on a row range
+    if Sq >= 4:
+        half = Sq // 2
+        sl = (slice(None), slice(half, None))
+        o2, l2 = od.clone(), ld.clone()
+        r2o, r2l = M.update_out_and_lse(o2, l2, bod[:, half:].contiguous(), bld[:, :, half:].contiguous(), slice_=sl)
+        assert r2o is o2 and r2l is l2
+        eo, el = O.merge_reference(out[sl], lse[sl], bo[:, half:], bl[:, :, half:])
+        assert torch.equal(o2.cpu()[:, :half], out[:, :half]) and torch.equal(l2.cpu()[:, :half], lse[:, :half])
+        assert torch.allclose(o2.cpu()[sl], eo, **TOL) and torch.allclose(l2.cpu()[sl], el, **TOL)
+    with pytest.raises(RuntimeError):
+        M.update_out_and_lse(None, None, bod, bld, slice_=(slice(None), slice(0, 1)))
+
+
+def test_merge_fused_final_epilogue():
+    import mercury_artifact_amd as M
+
+    B, Sq, H, D = 2, 70, 4, 128
+    out, lse, bo, bl = _blocks(B, Sq, H, D, seed=1)
+    ro, rl = O.merge_reference(out, lse, bo, bl)
+    fo = torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device="cuda")
+    fl = torch.empty(B, H, Sq, dtype=torch.float32, device="cuda")
+    M.merge_into(out.cuda(), lse.cuda(), bo.cuda(), bl.cuda(), None, None, fo, fl)
+    assert torch.allclose(fl.cpu(), rl.squeeze(-1).transpose(1, 2), **TOL)
+    # the bf16 cast of a value within 2e-6 of the reference differs by at most one bf16 ulp
+    assert (fo.float().cpu() - ro.bfloat16().float()).abs().max().item() <= 2 ** -7 * ro.abs().max().item()
+    frac_equal = (fo.cpu() == ro.bfloat16()).float().mean().item()
+    assert frac_equal > 0.999
+
+
+def test_merge_infinite_lse_is_identity():
+    import mercury_artifact_amd as M
+
+    B, Sq, H, D = 1, 16, 2, 128
+    out, lse, bo, bl = _blocks(B, Sq, H, D, seed=2)
+    ninf_b = torch.full_like(bl, -math.inf)
+    no, nl = M.update_out_and_lse(out.cuda(), lse.cuda(), bo.cuda(), ninf_b.cuda())
+    assert torch.equal(no.cpu(), out) and torch.equal(nl.cpu(), lse)
+    zo, zl = torch.zeros_like(out), torch.full_like(lse, -math.inf)
+    no, nl = M.update_out_and_lse(zo.cuda(), zl.cuda(), bo.cuda(), bl.cuda())
+    assert torch.equal(no.cpu(), bo.float()) and torch.equal(nl.cpu()[..., 0], bl.transpose(1, 2))
+    no, nl = M.update_out_and_lse(zo.cuda(), zl.cuda(), torch.zeros_like(bo).cuda(), ninf_b.cuda())
+    assert no.abs().max().item() == 0 and torch.isinf(nl).all() and not torch.isnan(no).any()
+
+
+@pytest.mark.parametrize("rows,D", [(64, 128), (37, 128), (3, 128), (50, 64), (7, 5)])
+def test_flash_reduce_and_pack(rows, D):
+    import mercury_artifact_amd as M
+
+    g = torch.Generator().manual_seed(rows)
+    lhs = torch.randn(1, rows, 1, D + 1, generator=g)
+    rhs = torch.randn(1, rows, 1, D + 1, generator=g)
+    lhs[..., -1] = lhs[..., -1] * 3 + 4
+    rhs[..., -1] = rhs[..., -1] * 3 + 4
+    ref = O.flash_reduce(lhs, rhs)
+    got = M.flash_reduce(lhs.cuda(), rhs.cuda())
+    assert got.shape == lhs.shape and torch.allclose(got.cpu(), ref, **TOL)
+    # pack, and pack fused with the reduce
+    bo = torch.randn(1, rows, 1, D, generator=g).bfloat16()
+    bl = torch.randn(1, 1, rows, generator=g) * 3 + 4
+    packed = M.pack_block(bo.cuda(), bl.cuda())
+    assert torch.equal(packed.cpu(), O.pack_block(bo, bl))
+    fused = M.pack_block(bo.cuda(), bl.cuda(), reduce_into=lhs.cuda())
+    assert torch.allclose(fused.cpu(), O.flash_reduce(lhs, O.pack_block(bo, bl)), **TOL)
+
+
+def test_pack_multi_head_layout():
+    import mercury_artifact_amd as M
+
+    B, Sq, H, D = 2, 11, 3, 128
+    _, _, bo, bl = _blocks(B, Sq, H, D, seed=4)
+    assert torch.equal(M.pack_block(bo.cuda(), bl.cuda()).cpu(), O.pack_block(bo, bl))
+
+
+@pytest.mark.parametrize("n", [4096, 1001, 3])
+def test_grad_accumulate(n):
+    import mercury_artifact_amd as M
+
+    g = torch.Generator().manual_seed(n)
+    acc = torch.randn(n, generator=g)
+    blk = torch.randn(n, generator=g).bfloat16()
+    assert torch.equal(M.grad_accumulate(None, blk.cuda()).cpu(), blk.float())
+    assert torch.equal(M.grad_accumulate(acc.cuda(), blk.cuda()).cpu(), acc + blk.float())

@@ -1,0 +1,135 @@
+"""Ring-step drivers on one GPU against the CPU oracle's ring step on the same seeded inputs.
+
+Same tolerances as the block kernel (bf16: max-abs(out) <= 2e-2, LSE rel <= 1e-3, own rel-L2 <= 1e-2);
+the reference's own tests accept max-abs < 1e-2 on out and lse (tests/test_search_validation.py:207-208),
+which is asserted too at the reference's test shape."""
+import pytest
+import torch
+
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(B, S, Hq, Hkv, D, W, seed=0):
+    """Full-sequence q, k, v (N(0,1) -> bf16) and the per-rank shards the reference's tests make with
+    ``chunk(W, dim=1)`` (example.py:161)."""
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, S, Hq, D, generator=g).bfloat16()
+    k = torch.randn(B, S, Hkv, D, generator=g).bfloat16()
+    v = torch.randn(B, S, Hkv, D, generator=g).bfloat16()
+    Sc = S // W
+    qs = [q[:, r * Sc:(r + 1) * Sc] for r in range(W)]
+    kvs = [torch.stack([k[:, r * Sc:(r + 1) * Sc], v[:, r * Sc:(r + 1) * Sc]]) for r in range(W)]
+    return q, k, v, qs, kvs
+
+
+def _compare(o, lse, ro, rl, out_atol=2e-2, lse_rtol=1e-3, rel_l2=1e-2):
+    o, lse = o.float().cpu(), lse.float().cpu()
+    assert (o - ro).abs().max().item() <= out_atol
+    assert (o - ro).norm().item() / ro.norm().item() <= rel_l2
+    assert ((lse - rl).abs() / rl.abs().clamp_min(1.0)).max().item() <= lse_rtol
+
+
+@pytest.mark.parametrize("rank", [0, 5])
+@pytest.mark.parametrize("fused", [False, True])
+def test_single_ring_reference_test_shape(rank, fused):
+    """B4 S4096 H5 D128 on an 8-rank ring (tests/test_ring_attn_codegen.py:84-87), one rank."""
+    import mercury_artifact_amd as M
+
+    B, S, H, D, W = 4, 4096, 5, 128, 8
+    q, k, v, qs, kvs = _inputs(B, S, H, H, D, W)
+    scale = D ** -0.5
+    ro, rl = O.single_pass_attention(qs[rank].float(), k.float(), v.float(), scale)
+    ring_o, ring_l = O.ring_forward(qs[rank].float(), [c.float() for c in kvs],
+                                    O.single_ring_order(rank, W), scale)
+    assert torch.allclose(ring_o, ro, atol=1e-5)           # oracle ring == oracle single pass
+    dev_kvs = [c.cuda() for c in kvs]
+    ring = M.LocalRing((W,), rank, dev_kvs)
+    qd = qs[rank].cuda()
+    o = torch.empty_like(qd)
+    lse = torch.empty(B, H, S // W, dtype=torch.float32, device="cuda")
+    q_before, kv_before = qd.clone(), dev_kvs[rank].clone()
+    M.flash_attn_pack_kv(qd, dev_kvs[rank], o, lse, scale, ring=ring, fused_epilogue=fused)
+    torch.cuda.synchronize()
+    _compare(o, lse, ring_o, ring_l)
+    assert (o.float().cpu() - ro).abs().max().item() < 1e-2 and (lse.cpu() - rl).abs().max().item() < 1e-2
+    assert torch.equal(qd, q_before) and torch.equal(dev_kvs[rank], kv_before)   # inputs untouched
+
+
+def test_gqa_ring():
+    """Hq 32 / Hkv 8 (tests/test_gqa.py:25), shortened sequence."""
+    import mercury_artifact_amd as M
+
+    B, S, Hq, Hkv, D, W, rank = 1, 2048, 32, 8, 128, 4, 2
+    q, k, v, qs, kvs = _inputs(B, S, Hq, Hkv, D, W, seed=1)
+    scale = D ** -0.5
+    ro, rl = O.ring_forward(qs[rank].float(), [c.float() for c in kvs], O.single_ring_order(rank, W), scale)
+    dev = [c.cuda() for c in kvs]
+    o = torch.empty(B, S // W, Hq, D, dtype=torch.bfloat16, device="cuda")
+    lse = torch.empty(B, Hq, S // W, dtype=torch.float32, device="cuda")
+    M.gqa_pack_kv(qs[rank].cuda(), dev[rank], o, lse, scale, ring=M.LocalRing((W,), rank, dev))
+    _compare(o, lse, ro, rl)
+
+
+@pytest.mark.parametrize("rank", [0, 6])
+def test_double_ring(rank):
+    """(inner, outer) = (4, 2) mesh (tests/test_double_ring.py:56)."""
+    import mercury_artifact_amd as M
+
+    B, S, H, D, W = 1, 2048, 4, 128, 8
+    q, k, v, qs, kvs = _inputs(B, S, H, H, D, W, seed=2)
+    scale = D ** -0.5
+    order = O.double_ring_order(rank, 4, 2)
+    ro, rl = O.ring_forward(qs[rank].float(), [c.float() for c in kvs], order, scale)
+    dev = [c.cuda() for c in kvs]
+    ring = M.LocalRing((4, 2), rank, dev)
+    seen = []
+    real_send = ring.send_recv
+
+    def spy(*a, **kw):
+        got = real_send(*a, **kw)
+        seen.append(ring.current)
+        return got
+    ring.send_recv = spy
+    o = torch.empty(B, S // W, H, D, dtype=torch.bfloat16, device="cuda")
+    lse = torch.empty(B, H, S // W, dtype=torch.float32, device="cuda")
+    M.flash_attn_pack_split_kv(qs[rank].cuda(), dev[rank], o, lse, scale, ring=ring)
+    assert [rank] + seen == order
+    _compare(o, lse, ro, rl)
+
+
+def test_packed_reduce_ring():
+    import mercury_artifact_amd as M
+
+    B, S, H, D, W, rank = 2, 1024, 3, 128, 4, 1
+    q, k, v, qs, kvs = _inputs(B, S, H, H, D, W, seed=3)
+    scale = D ** -0.5
+    ro, rl = O.ring_forward_packed(qs[rank].float(), [c.float() for c in kvs], O.single_ring_order(rank, W), scale)
+    dev = [c.cuda() for c in kvs]
+    o = torch.empty(B, S // W, H, D, dtype=torch.bfloat16, device="cuda")
+    lse = torch.empty(B, H, S // W, dtype=torch.float32, device="cuda")
+    M.flash_attn_expose_reduce(qs[rank].cuda(), dev[rank], o, lse, scale, ring=M.LocalRing((W,), rank, dev))
+    _compare(o, lse, ro, rl)
+
+
+@pytest.mark.parametrize("rank", [0, 1, 3])
+def test_zigzag_causal_ring(rank):
+    """Causal GQA in the zigzag layout, scaled-down BASELINE configs[2] (B2 Hq32/Hkv8 D128)."""
+    import mercury_artifact_amd as M
+
+    B, Hq, Hkv, D, W, block = 2, 8, 2, 128, 4, 192
+    S = 2 * W * block
+    g = torch.Generator().manual_seed(4)
+    q = torch.randn(B, S, Hq, D, generator=g).bfloat16()
+    k = torch.randn(B, S, Hkv, D, generator=g).bfloat16()
+    v = torch.randn(B, S, Hkv, D, generator=g).bfloat16()
+    scale = D ** -0.5
+    ref_o, ref_l = O.single_pass_attention(q.float(), k.float(), v.float(), scale, causal=True)
+    pos = [O.zigzag_local_positions(r, W, block) for r in range(W)]
+    dev = [torch.stack([k[:, p], v[:, p]]).cuda() for p in pos]
+    qd = q[:, pos[rank]].cuda()
+    o = torch.empty_like(qd)
+    lse = torch.empty(B, Hq, 2 * block, dtype=torch.float32, device="cuda")
+    M.zigzag_causal_pack_kv(qd, dev[rank], o, lse, scale, ring=M.LocalRing((W,), rank, dev))
+    _compare(o, lse, ref_o[:, pos[rank]], ref_l[:, :, pos[rank]])
