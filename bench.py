@@ -1,0 +1,170 @@
+#!/usr/bin/env python3
+"""Headline benchmark: one rank's bf16 ring-attention forward step on one MI355X.
+
+Workload = BASELINE.json configs[1]: batch 1, 32 heads, head dim 128, local Q of 4096 rows, 8 KV chunks
+of 4096 rows (32768 keys), non-causal, N(0,1) inputs cast to bf16, softmax scale 128^-0.5.
+A step = 8 block-forward kernels + the first-call cast + 7 LSE merges + the bf16 / (B,H,S) epilogue,
+driven through the same operators Mercury's generated code calls.  Inputs are resident in HBM before
+the timed region.  Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+
+
+def cpu_baseline(sample_heads: int, B: int, Sq: int, D: int, W: int):
+    """The fp32 oracle (a CPU port of the same step) on `sample_heads` of the 32 heads."""
+    import torch
+
+    import oracle as O
+
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(B, Sq, sample_heads, D, generator=g)
+    kvs = [torch.randn(2, B, Sq, sample_heads, D, generator=g) for _ in range(W)]
+    scale = D ** -0.5
+    order = O.single_ring_order(0, W)
+    O.ring_forward(q[:, :256], [c[:, :, :256] for c in kvs], order, scale)      # warm-up
+    t0 = time.perf_counter()
+    O.ring_forward(q, kvs, order, scale)
+    dt = time.perf_counter() - t0
+    flops = 4.0 * B * sample_heads * Sq * Sq * D * W
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{sample_heads} of 32 heads of the same step (Q 4096 x 8 chunks of 4096, fp32 torch "
+                      f"matmul/logsumexp + merge), {dt:.1f} s"}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--cpu-heads", type=int, default=4, help="heads in the CPU baseline sample (0 = skip)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one rank's step on ONE GPU (the ring is emulated by local buffer rotation); "
+              "--gpus must be 1", file=sys.stderr)
+        return 2
+
+    import torch
+
+    import mercury_artifact_amd as M
+    from mercury_artifact_amd import flash_attn_interface as FI
+    from mercury_artifact_amd import merge as MG
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    B, Sq, H, D, W, rank = 1, 4096, 32, 128, 8, 0
+    torch.manual_seed(0)
+    q = torch.randn(B, Sq, H, D).bfloat16().to(dev)
+    kvs = [torch.randn(2, B, Sq, H, D).bfloat16().to(dev) for _ in range(W)]
+    o = torch.empty_like(q)
+    lse = torch.empty(B, H, Sq, dtype=torch.float32, device=dev)
+    scale = D ** -0.5
+
+    # per-kernel durations: HIP events on the stream the kernels are launched on (torch's current one)
+    fwd_events, merge_events = [], []
+    real_fwd, real_merge = FI.attn_fwd_block, MG.merge_into
+    recording = {"on": False}
+
+    def timed(real, bucket):
+        def wrapper(*a, **kw):
+            if not recording["on"]:
+                return real(*a, **kw)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            r = real(*a, **kw)
+            e1.record()
+            bucket.append((e0, e1, a, kw))
+            return r
+        return wrapper
+
+    FI.attn_fwd_block = timed(real_fwd, fwd_events)
+    MG.merge_into = timed(real_merge, merge_events)
+
+    def step(fused=False):
+        ring = M.LocalRing((W,), rank, kvs)
+        M.flash_attn_pack_kv(q, kvs[rank], o, lse, scale, ring=ring, fused_epilogue=fused)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    recording["on"] = True
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    recording["on"] = False
+
+    ms_per_step = dt / args.steps * 1e3
+    flops_per_block = 4.0 * B * H * Sq * Sq * D
+    flops_per_step = flops_per_block * W
+    value = flops_per_step / (ms_per_step * 1e-3) / 1e12
+
+    fwd_ms = sum(e0.elapsed_time(e1) for e0, e1, _, _ in fwd_events) / max(len(fwd_events), 1)
+    fwd_tflops = flops_per_block / (fwd_ms * 1e-3) / 1e12
+    rows = B * Sq * H
+    merge_bytes = rows * (D * 10 + 12)
+    real_merges = [(e0, e1) for e0, e1, a, _ in merge_events if a[0] is not None]
+    merge_ms = sum(e0.elapsed_time(e1) for e0, e1 in real_merges) / max(len(real_merges), 1)
+    merge_gbs = merge_bytes / (merge_ms * 1e-3) / 1e9
+
+    # the same step with the last merge writing o / lse directly (identical arithmetic)
+    for _ in range(2):
+        step(True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(True)
+    torch.cuda.synchronize()
+    fused_ms = (time.perf_counter() - t0) / args.steps * 1e3
+
+    props = torch.cuda.get_device_properties(0)
+    result = {
+        "metric": "per-rank ring-attn step TFLOP/s + % MFMA peak (bf16, d128, Q 4096 x 8 chunks)",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE configs[1]: bf16 non-causal MHA, B1 H32 D128, local Q 4096 x 8 KV chunks "
+                               "of 4096 (single ring, rank 0), 8 block forwards + 7 LSE merges + epilogue",
+                   "flops_per_step": flops_per_step, "pct_of_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
+                   "fused_epilogue_ms_per_step": round(fused_ms, 4),
+                   "device": props.gcnArchName, "cus": props.multi_processor_count},
+        "roofline": {"bound": "mfma", "kernel": "attn_fwd_bf16_d128", "achieved": round(fwd_tflops, 2),
+                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(fwd_tflops / PEAK_BF16_TFLOPS, 4),
+                     "traffic": None, "avg_launch_ms": round(fwd_ms, 4), "launches": len(fwd_events)},
+        "roofline_merge": {"bound": "hbm", "kernel": "lse_merge_kernel", "achieved": round(merge_gbs, 1),
+                           "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(merge_gbs / PEAK_HBM_GBS, 4),
+                           "traffic": None, "avg_launch_ms": round(merge_ms, 5), "launches": len(real_merges),
+                           "bytes_per_launch": merge_bytes},
+    }
+    if args.cpu_heads > 0:
+        result["cpu_baseline"] = cpu_baseline(args.cpu_heads, B, Sq, D, W)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

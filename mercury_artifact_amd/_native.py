@@ -12,7 +12,9 @@ from typing import Optional
 
 import torch
 
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libmercury_hip.so")
+# MERCURY_HIP_LIB points at another build of the same library (e.g. one compiled with other tuning macros).
+LIB_PATH = os.environ.get("MERCURY_HIP_LIB") or os.path.join(
+    os.path.dirname(os.path.abspath(__file__)), "csrc", "libmercury_hip.so")
 
 MHIP_BF16, MHIP_E4M3 = 0, 1
 MASK_NONE, MASK_CAUSAL = 0, 1

@@ -6,8 +6,6 @@ namespace mhip {
 int attn_fwd_bf16(const void* q, const void* k, const void* v, void* out, float* lse,
                   int B, int Sq, int Sc, int Hq, int Hkv,
                   const int64_t* strides, float scale, int mask, hipStream_t stream);
-int fill_empty_block(void* out, float* lse, int B, int Sq, int Hq, int D,
-                     int64_t o_sb, int64_t o_ss, int64_t o_sh, hipStream_t stream);
 }  // namespace mhip
 
 using namespace mhip;
@@ -56,6 +54,9 @@ extern "C" int mhip_attn_fwd_block(const void* q, const void* k, const void* v, 
   if (!mult8(q_sb) || !mult8(q_ss) || !mult8(q_sh) || !mult8(k_sb) || !mult8(k_ss) || !mult8(k_sh) ||
       !mult8(v_sb) || !mult8(v_ss) || !mult8(v_sh) || !mult8(o_sb) || !mult8(o_ss) || !mult8(o_sh))
     return MHIP_EALIGN;
+  // K / V tiles are fetched through 32-bit buffer offsets relative to the (batch, head) base
+  const int64_t kv_span = (int64_t)Sc * (k_ss > v_ss ? k_ss : v_ss) * 2;
+  if (k_ss < 0 || v_ss < 0 || kv_span >= (int64_t(1) << 31)) return MHIP_EUNSUPPORTED;
   const int64_t strides[12] = {q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, v_sb, v_ss, v_sh, o_sb, o_ss, o_sh};
   return attn_fwd_bf16(q, k, v, out, lse, B, Sq, Sc, Hq, Hkv, strides, softmax_scale, mask, st);
 }

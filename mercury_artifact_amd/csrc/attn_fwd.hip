@@ -4,7 +4,7 @@
 // Replaces the flash-attn call at utils/flash_attn_dsl.py:159-176 of the reference.
 //
 // Work decomposition
-//   workgroup  = 128 Q rows of one (batch, q-head): 4 wavefronts x 32 rows, two workgroups per CU
+//   workgroup  = 256 Q rows of one (batch, q-head): 8 wavefronts x 32 rows, one workgroup per CU
 //   main loop  = 64-key tiles of the chunk, K and V double-buffered in LDS
 //   S^T = K Q^T  : v_mfma_f32_32x32x16_bf16 with A = K rows (LDS), B = Q (registers, loaded once).
 //                  The accumulator layout puts one Q row in each lane (lane % 32) and 32 of the
@@ -20,9 +20,7 @@ namespace mhip {
 namespace {
 
 constexpr int kD = 128;            // head dimension
-constexpr int kBM = 128;           // Q rows per workgroup
 constexpr int kBN = 64;            // keys per main-loop tile
-constexpr int kThreads = 256;
 constexpr int kKStride = kD + 8;   // bf16 elements per K row in LDS (272 B: 16 B skew per row)
 constexpr int kVStride = kBN + 8;  // bf16 elements per V^T row in LDS (144 B)
 constexpr int kKBytes = kBN * kKStride * 2;   // 17408
@@ -36,13 +34,24 @@ struct FwdParams {
   int B, Sq, Sc, Hq, Hkv, group;
   int64_t q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, v_sb, v_ss, v_sh, o_sb, o_ss, o_sh;
   float scale, scale_log2;
-  int nq_tiles;      // ceil(Sq / 128)
+  int nq_tiles;      // ceil(Sq / rows per workgroup)
   int total;         // B * Hq * nq_tiles
   int per_xcd;       // ceil(total / 8)
 };
 
-template <bool CAUSAL>
-__global__ __launch_bounds__(kThreads, 2) void attn_fwd_bf16_d128(const FwdParams p) {
+// Buffer descriptor over `bytes` bytes at `base`: loads past the end return zero, so rows beyond the
+// chunk need no address clamping (their scores are masked afterwards).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+// PIPE: the S^T MFMAs of tile t+1 are issued before the softmax of tile t so that the matrix pipe has
+// work while the VALU does the exponentials.
+// NW: wavefronts per workgroup (32 Q rows each).  With 8, wavefronts 0-3 stage the K tile and 4-7
+// the V tile, so one copy of each tile in LDS serves 256 Q rows.
+template <bool CAUSAL, bool PIPE, int NW>
+__global__ __launch_bounds__(NW * 64, 2) void attn_fwd_bf16_d128(const FwdParams p) {
+  constexpr int kBM = NW * 32;
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kStageBytes];
 
   // Workgroup i runs on XCD i % 8.  Give every XCD a contiguous range of the (batch, head, q-tile)
@@ -85,35 +94,49 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_bf16_d128(const FwdParam
   // ---- global -> register staging of one K/V tile ---------------------------------------------
   // K: thread loads rows (tid/16 + 16 i), 16-byte chunk tid%16.
   // V: thread loads the four rows of key quad tid/16, chunk tid%16 (8 head-dim values each).
+  // Per-thread byte offsets are fixed; the tile advances through the scalar offset of the load.
+  const bool does_k = NW == 4 || wave < 4;
+  const bool does_v = NW == 4 || wave >= 4;
   const int ld_chunk = tid & 15;
-  const int ld_row = tid >> 4;
-  const uint16_t* kbase = p.k + b * p.k_sb + hk * p.k_sh + ld_chunk * 8;
-  const uint16_t* vbase = p.v + b * p.v_sb + hk * p.v_sh + ld_chunk * 8;
+  const int ld_row = (tid & 255) >> 4;
+  const __amdgpu_buffer_rsrc_t krs =
+      make_rsrc(p.k + b * p.k_sb + hk * p.k_sh, (uint32_t)(((int64_t)(p.Sc - 1) * p.k_ss + kD) * 2));
+  const __amdgpu_buffer_rsrc_t vrs =
+      make_rsrc(p.v + b * p.v_sb + hk * p.v_sh, (uint32_t)(((int64_t)(p.Sc - 1) * p.v_ss + kD) * 2));
+  int koff[4], voff[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    koff[i] = (int)((ld_row + 16 * i) * p.k_ss * 2) + ld_chunk * 16;
+    voff[i] = (int)((ld_row * 4 + i) * p.v_ss * 2) + ld_chunk * 16;
+  }
+  const int k_tile_bytes = (int)(kBN * p.k_ss * 2);
+  const int v_tile_bytes = (int)(kBN * p.v_ss * 2);
   u32x4 kreg[4], vreg[4];
 
-  auto load_tile = [&](int t) {
-    const int kv0 = t * kBN;
+  auto load_k = [&](int t) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      int rk = kv0 + ld_row + 16 * i;
-      rk = rk < p.Sc ? rk : p.Sc - 1;
-      kreg[i] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)rk * p.k_ss);
-      int rv = kv0 + ld_row * 4 + i;
-      rv = rv < p.Sc ? rv : p.Sc - 1;
-      vreg[i] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)rv * p.v_ss);
-    }
+    for (int i = 0; i < 4; ++i) kreg[i] = __builtin_amdgcn_raw_buffer_load_b128(krs, koff[i], t * k_tile_bytes, 0);
+  };
+  auto load_v = [&](int t) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) vreg[i] = __builtin_amdgcn_raw_buffer_load_b128(vrs, voff[i], t * v_tile_bytes, 0);
   };
 
   // LDS position of key quad (4 consecutive keys) inside a V^T row: MFMA k-step = quad / 4,
   // lane half = quad % 2, first / second group of four accumulator registers = (quad % 4) / 2.
   const int vt_off = ((ld_row >> 2) * 2 + (ld_row & 1)) * 16 + ((ld_row & 3) >> 1) * 8;
+  // Row d of V^T lives in LDS row d ^ rev3(d >> 4): the 16 lanes of one write (rows 8c + e, c = 0..15)
+  // and the 32 lanes of one read (rows 32 db + 0..31) then both spread over all banks.
+  const int vt_xor = ((ld_chunk >> 3) & 1) | (((ld_chunk >> 2) & 1) << 1) | (((ld_chunk >> 1) & 1) << 2);
 
-  auto store_tile = [&](int stage) {
+  auto store_k = [&](int stage) {
     unsigned char* ks = smem + stage * kStageBytes;
-    unsigned char* vs = ks + kKBytes;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       *reinterpret_cast<u32x4*>(ks + (ld_row + 16 * i) * (kKStride * 2) + ld_chunk * 16) = kreg[i];
+  };
+  auto store_v = [&](int stage) {
+    unsigned char* vs = smem + stage * kStageBytes + kKBytes;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       // dword j of each row holds head-dim values 2j (low half) and 2j+1 (high half)
@@ -122,39 +145,25 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_bf16_d128(const FwdParam
       even[1] = __builtin_amdgcn_perm(vreg[3][j], vreg[2][j], 0x05040100u);
       odd[0] = __builtin_amdgcn_perm(vreg[1][j], vreg[0][j], 0x07060302u);
       odd[1] = __builtin_amdgcn_perm(vreg[3][j], vreg[2][j], 0x07060302u);
-      const int d = ld_chunk * 8 + 2 * j;
-      *reinterpret_cast<u32x2*>(vs + d * (kVStride * 2) + vt_off) = even;
-      *reinterpret_cast<u32x2*>(vs + (d + 1) * (kVStride * 2) + vt_off) = odd;
+      const int r0 = ld_chunk * 8 + ((2 * j) ^ vt_xor);
+      const int r1 = ld_chunk * 8 + ((2 * j + 1) ^ vt_xor);
+      *reinterpret_cast<u32x2*>(vs + r0 * (kVStride * 2) + vt_off) = even;
+      *reinterpret_cast<u32x2*>(vs + r1 * (kVStride * 2) + vt_off) = odd;
     }
   };
 
-  // ---- accumulators -----------------------------------------------------------------------------
-  f32x16 o_acc[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 16; ++j) o_acc[i][j] = 0.f;
-  float m_run = -INFINITY;   // running max of the raw (unscaled) scores of this lane's Q row
-  float l_run = 0.f;         // this lane's share of the running sum (the other 32 keys: lane ^ 32)
-
   const int k_rd = ln * (kKStride * 2) + hf * 16;   // + mb*32*272 + ks*32
-  const int v_rd = ln * (kVStride * 2) + hf * 16;   // + db*32*144 + kstep*32
+  int v_rd[4];                                        // + kstep*32
+#pragma unroll
+  for (int db = 0; db < 4; ++db) {
+    const int x = (db >> 1) | ((db & 1) << 1) | ((ln >> 4) << 2);
+    v_rd[db] = (db * 32 + (ln ^ x)) * (kVStride * 2) + hf * 16;
+  }
   const int causal_shift = p.Sc - p.Sq;
 
-  if (ntiles > 0) {
-    load_tile(0);
-    store_tile(0);
-  }
-
-  for (int t = 0; t < ntiles; ++t) {
-    const int stage = t & 1;
-    if (t + 1 < ntiles) load_tile(t + 1);
-    __syncthreads();
+  // S^T tile: 64 keys x 32 q rows per wave
+  auto qk = [&](int stage, f32x16 (&s)[2]) {
     const unsigned char* ks = smem + stage * kStageBytes;
-    const unsigned char* vs = ks + kKBytes;
-
-    // ---- S^T tile: 64 keys x 32 q rows per wave ---------------------------------------------------
-    f32x16 s[2];
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
@@ -166,6 +175,51 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_bf16_d128(const FwdParam
         const bf16x8 kf = *reinterpret_cast<const bf16x8*>(ks + k_rd + mb * (32 * kKStride * 2) + kk * 32);
         s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], s[mb], 0, 0, 0);
       }
+    }
+  };
+
+  // ---- accumulators -----------------------------------------------------------------------------
+  f32x16 o_acc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) o_acc[i][j] = 0.f;
+  // m_ref: the score (raw, unscaled) the exponentials of this lane's Q row are taken relative to.  It
+  // follows the running maximum lazily: it only moves when the maximum has grown by more than
+  // kRescaleSlack (in log2 units of the scaled score), so exp2 arguments stay below that slack and the
+  // O accumulator is rescaled on few tiles.  The LSE does not depend on the choice of reference.
+  float m_ref = -INFINITY;
+  float l_run = 0.f;         // this lane's share of the running sum (the other 32 keys: lane ^ 32)
+  constexpr float kRescaleSlack = 8.f;
+
+  f32x16 s_cur[2], s_nxt[2];
+
+  if (ntiles > 0) {
+    if (does_k) { load_k(0); store_k(0); }
+    if (does_v) { load_v(0); store_v(0); }
+    if (PIPE) {
+      if (does_k && ntiles > 1) { load_k(1); store_k(1); }
+      __syncthreads();
+      qk(0, s_cur);
+    }
+  }
+
+  for (int t = 0; t < ntiles; ++t) {
+    const int stage = t & 1;
+    if (PIPE) {
+      if (does_k && t + 2 < ntiles) load_k(t + 2);
+      if (does_v && t + 1 < ntiles) load_v(t + 1);
+    } else if (t + 1 < ntiles) {
+      if (does_k) load_k(t + 1);
+      if (does_v) load_v(t + 1);
+    }
+    __syncthreads();
+    const unsigned char* vs = smem + stage * kStageBytes + kKBytes;
+
+    if (PIPE) {
+      if (t + 1 < ntiles) qk(stage ^ 1, s_nxt);
+    } else {
+      qk(stage, s_cur);
     }
 
     // ---- mask: keys past the chunk end, and the causal diagonal ---------------------------------
@@ -180,36 +234,41 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_bf16_d128(const FwdParam
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
           const int key = kv0 + mb * 32 + (j >> 2) * 8 + hf * 4 + (j & 3);
-          if (key > lim) s[mb][j] = -INFINITY;
+          if (key > lim) s_cur[mb][j] = -INFINITY;
         }
     }
 
     // ---- online softmax (per lane = per Q row) ----------------------------------------------------
-    float mx = s[0][0];
+    float mx = s_cur[0][0];
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-      for (int j = 0; j < 16; ++j) mx = fmaxf(mx, s[mb][j]);
+      for (int j = 0; j < 16; ++j) mx = fmaxf(mx, s_cur[mb][j]);
     mx = pair_max(mx);
-    const float m_new = fmaxf(m_run, mx);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = fast_exp2((m_run - m_use) * p.scale_log2);
-    const float msc = m_use * p.scale_log2;
-    m_run = m_new;
+    // move the reference only when the maximum outgrew it by the slack (always on the first tile
+    // that has a visible key: m_ref = -inf there)
+    const bool grow = (mx - m_ref) * p.scale_log2 > kRescaleSlack;     // false for NaN (-inf - -inf)
+    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+      const float m_new = grow ? mx : m_ref;
+      const float alpha = (m_new == -INFINITY) ? 1.f : fast_exp2((m_ref - m_new) * p.scale_log2);
+      m_ref = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) o_acc[db][j] *= alpha;
+    }
+    const float msc = (m_ref == -INFINITY) ? 0.f : m_ref * p.scale_log2;
     float rs = 0.f;
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
-        const float e = fast_exp2(__builtin_fmaf(s[mb][j], p.scale_log2, -msc));
-        s[mb][j] = e;
+        const float e = fast_exp2(__builtin_fmaf(s_cur[mb][j], p.scale_log2, -msc));
+        s_cur[mb][j] = e;
         rs += e;
       }
-    l_run = l_run * alpha + rs;
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-      for (int j = 0; j < 16; ++j) o_acc[db][j] *= alpha;
+    l_run += rs;
 
     // ---- P^T as bf16 B operands: k-step (mb, j2) takes accumulator registers 8 j2 .. 8 j2 + 7 ---
     bf16x8 pf[4];
@@ -219,7 +278,8 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_bf16_d128(const FwdParam
       for (int j2 = 0; j2 < 2; ++j2) {
         u32x4 w;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) w[e] = pack_bf16(s[mb][8 * j2 + 2 * e], s[mb][8 * j2 + 2 * e + 1]);
+        for (int e = 0; e < 4; ++e)
+          w[e] = pack_bf16(s_cur[mb][8 * j2 + 2 * e], s_cur[mb][8 * j2 + 2 * e + 1]);
         pf[mb * 2 + j2] = __builtin_bit_cast(bf16x8, w);
       }
 
@@ -228,19 +288,27 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_bf16_d128(const FwdParam
     for (int kstep = 0; kstep < 4; ++kstep) {
 #pragma unroll
       for (int db = 0; db < 4; ++db) {
-        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vs + v_rd + db * (32 * kVStride * 2) + kstep * 32);
+        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vs + v_rd[db] + kstep * 32);
         o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kstep], o_acc[db], 0, 0, 0);
       }
     }
 
-    if (t + 1 < ntiles) store_tile(stage ^ 1);
+    if (PIPE) {
+      if (does_k && t + 2 < ntiles) store_k(stage);
+      if (does_v && t + 1 < ntiles) store_v(stage ^ 1);
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) s_cur[mb] = s_nxt[mb];
+    } else if (t + 1 < ntiles) {
+      if (does_k) store_k(stage ^ 1);
+      if (does_v) store_v(stage ^ 1);
+    }
   }
 
   // ---- epilogue -----------------------------------------------------------------------------------
   const float l_tot = pair_sum(l_run);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   if (hf == 0 && my_q < p.Sq) {
-    const float lse = l_tot > 0.f ? m_run * p.scale + fast_log2(l_tot) * kLn2 : -INFINITY;
+    const float lse = l_tot > 0.f ? m_ref * p.scale + fast_log2(l_tot) * kLn2 : -INFINITY;
     p.lse[((int64_t)b * p.Hq + hq) * p.Sq + my_q] = lse;
   }
 
@@ -289,14 +357,21 @@ int attn_fwd_bf16(const void* q, const void* k, const void* v, void* out, float*
   p.o_sb = st[9]; p.o_ss = st[10]; p.o_sh = st[11];
   p.scale = scale;
   p.scale_log2 = scale * kLog2e;
+#ifndef MHIP_FWD_PIPE
+#define MHIP_FWD_PIPE false
+#endif
+#ifndef MHIP_FWD_WAVES
+#define MHIP_FWD_WAVES 8
+#endif
+  constexpr int kBM = MHIP_FWD_WAVES * 32;
   p.nq_tiles = (Sq + kBM - 1) / kBM;
   p.total = B * Hq * p.nq_tiles;
   p.per_xcd = (p.total + 7) / 8;
-  const dim3 grid(p.per_xcd * 8), block(kThreads);
+  const dim3 grid(p.per_xcd * 8), block(MHIP_FWD_WAVES * 64);
   if (mask == MHIP_MASK_CAUSAL)
-    hipLaunchKernelGGL(attn_fwd_bf16_d128<true>, grid, block, 0, stream, p);
+    hipLaunchKernelGGL((attn_fwd_bf16_d128<true, MHIP_FWD_PIPE, MHIP_FWD_WAVES>), grid, block, 0, stream, p);
   else
-    hipLaunchKernelGGL(attn_fwd_bf16_d128<false>, grid, block, 0, stream, p);
+    hipLaunchKernelGGL((attn_fwd_bf16_d128<false, MHIP_FWD_PIPE, MHIP_FWD_WAVES>), grid, block, 0, stream, p);
   return launch_status();
 }
 
