@@ -4,8 +4,10 @@
 // Replaces the flash-attn call at utils/flash_attn_dsl.py:159-176 of the reference.
 //
 // Work decomposition
-//   workgroup  = 256 Q rows of one (batch, q-head): 8 wavefronts x 32 rows, one workgroup per CU
-//   main loop  = 64-key tiles of the chunk, K and V double-buffered in LDS
+//   workgroup  = 256 Q rows of one (batch, q-head): 8 wavefronts x 32 rows, one workgroup per CU,
+//                two wavefronts per SIMD
+//   main loop  = 64-key tiles of the chunk, K and V double-buffered in LDS; wavefronts 0-3 stage K,
+//                wavefronts 4-7 stage V (transposed in registers with v_perm_b32 on the way)
 //   S^T = K Q^T  : v_mfma_f32_32x32x16_bf16 with A = K rows (LDS), B = Q (registers, loaded once).
 //                  The accumulator layout puts one Q row in each lane (lane % 32) and 32 of the
 //                  64 keys of the tile in that lane's registers, so the online softmax needs one
@@ -13,13 +15,21 @@
 //   O^T = V^T P^T: the same lane that produced P^T[key][q] feeds it back as the B operand; the
 //                  key order inside one MFMA k-step is whatever the accumulator registers hold,
 //                  and V^T is written to LDS in exactly that key order, so P never moves.
-//   V^T          : transposed in registers (v_perm_b32) on its way from global memory to LDS.
+//   ping-pong    : every tile is split into a matrix phase (S^T of the next tile + O^T of this one,
+//                  32 MFMAs) and a vector phase (softmax of the next tile, LDS stores).  Wavefronts
+//                  0-3 and 4-7 run half a tile apart, separated by workgroup barriers, so on every
+//                  SIMD one wavefront feeds the matrix pipe while the other does exponentials.
 #include "mhip_common.hpp"
+#ifdef MHIP_FWD_TRACE
+#include <cstdlib>
+#endif
 
 namespace mhip {
 namespace {
 
 constexpr int kD = 128;            // head dimension
+constexpr int kWaves = 8;
+constexpr int kBM = kWaves * 32;   // Q rows per workgroup
 constexpr int kBN = 64;            // keys per main-loop tile
 constexpr int kKStride = kD + 8;   // bf16 elements per K row in LDS (272 B: 16 B skew per row)
 constexpr int kVStride = kBN + 8;  // bf16 elements per V^T row in LDS (144 B)
@@ -27,6 +37,14 @@ constexpr int kKBytes = kBN * kKStride * 2;   // 17408
 constexpr int kVBytes = kD * kVStride * 2;    // 18432
 constexpr int kStageBytes = kKBytes + kVBytes;
 constexpr int kOStride = kD + 8;   // epilogue staging of O, bf16 elements per row
+#ifndef MHIP_FWD_PINGPONG
+#define MHIP_FWD_PINGPONG 1
+#endif
+#ifndef MHIP_FWD_FRAG_DEPTH
+#define MHIP_FWD_FRAG_DEPTH 8
+#endif
+constexpr int kFragDepth = MHIP_FWD_FRAG_DEPTH;  // LDS operand reads in flight ahead of the MFMAs
+constexpr bool kPingPong = MHIP_FWD_PINGPONG;   // 0: all wavefronts run the phases in lock step
 
 struct FwdParams {
   const uint16_t* q; const uint16_t* k; const uint16_t* v;
@@ -37,6 +55,9 @@ struct FwdParams {
   int nq_tiles;      // ceil(Sq / rows per workgroup)
   int total;         // B * Hq * nq_tiles
   int per_xcd;       // ceil(total / 8)
+#ifdef MHIP_FWD_TRACE
+  long long* trace;
+#endif
 };
 
 // Buffer descriptor over `bytes` bytes at `base`: loads past the end return zero, so rows beyond the
@@ -45,14 +66,16 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
 }
 
-// PIPE: the S^T MFMAs of tile t+1 are issued before the softmax of tile t so that the matrix pipe has
-// work while the VALU does the exponentials.
-// NW: wavefronts per workgroup (32 Q rows each).  With 8, wavefronts 0-3 stage the K tile and 4-7
-// the V tile, so one copy of each tile in LDS serves 256 Q rows.
-template <bool CAUSAL, bool PIPE, int NW>
-__global__ __launch_bounds__(NW * 64, 2) void attn_fwd_bf16_d128(const FwdParams p) {
-  constexpr int kBM = NW * 32;
+template <bool CAUSAL>
+__global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdParams p) {
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kStageBytes];
+#ifdef MHIP_FWD_TRACE
+  __shared__ long long tr_buf[8 * 400];
+  int tr_n = 0;
+#define TR() do { if (blockIdx.x == 0 && tr_n < 400) { tr_buf[(threadIdx.x >> 6) * 400 + tr_n] = clock64(); } ++tr_n; } while (0)
+#else
+#define TR() do {} while (0)
+#endif
 
   // Workgroup i runs on XCD i % 8.  Give every XCD a contiguous range of the (batch, head, q-tile)
   // order so that the workgroups sharing one K/V head also share one L2.
@@ -67,10 +90,11 @@ __global__ __launch_bounds__(NW * 64, 2) void attn_fwd_bf16_d128(const FwdParams
   const int q0 = qt * kBM;
 
   const int tid = threadIdx.x;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: role branches stay uniform
   const int lane = tid & 63;
   const int ln = lane & 31;
   const int hf = lane >> 5;
+  const bool group_b = wave >= 4;                 // second ping-pong group; these waves stage V
 
   // ---- number of key tiles this Q tile has to visit -------------------------------------------
   int kv_end = p.Sc;
@@ -89,37 +113,31 @@ __global__ __launch_bounds__(NW * 64, 2) void attn_fwd_bf16_d128(const FwdParams
     const uint16_t* qp = p.q + b * p.q_sb + (int64_t)row * p.q_ss + hq * p.q_sh + hf * 8;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qp + ks * 16);
+    // Pin the fragment here: otherwise its first use sits inside the main loop and the wait for
+    // these loads lands there, where it also waits for the tile prefetch issued just before it.
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) asm volatile("" : "+v"(qf[ks]));
   }
 
-  // ---- global -> register staging of one K/V tile ---------------------------------------------
-  // K: thread loads rows (tid/16 + 16 i), 16-byte chunk tid%16.
-  // V: thread loads the four rows of key quad tid/16, chunk tid%16 (8 head-dim values each).
+  // ---- global -> register staging of one K or V tile ----------------------------------------------
+  // K (waves 0-3): thread loads rows (lt/16 + 16 i), 16-byte chunk lt%16, lt = tid % 256.
+  // V (waves 4-7): thread loads the four rows of key quad lt/16, chunk lt%16 (8 head-dim values each).
   // Per-thread byte offsets are fixed; the tile advances through the scalar offset of the load.
-  const bool does_k = NW == 4 || wave < 4;
-  const bool does_v = NW == 4 || wave >= 4;
   const int ld_chunk = tid & 15;
   const int ld_row = (tid & 255) >> 4;
-  const __amdgpu_buffer_rsrc_t krs =
-      make_rsrc(p.k + b * p.k_sb + hk * p.k_sh, (uint32_t)(((int64_t)(p.Sc - 1) * p.k_ss + kD) * 2));
-  const __amdgpu_buffer_rsrc_t vrs =
-      make_rsrc(p.v + b * p.v_sb + hk * p.v_sh, (uint32_t)(((int64_t)(p.Sc - 1) * p.v_ss + kD) * 2));
-  int koff[4], voff[4];
+  const uint16_t* gbase = group_b ? p.v + b * p.v_sb + hk * p.v_sh : p.k + b * p.k_sb + hk * p.k_sh;
+  const int64_t g_ss = group_b ? p.v_ss : p.k_ss;
+  const __amdgpu_buffer_rsrc_t grs = make_rsrc(gbase, (uint32_t)(((int64_t)(p.Sc - 1) * g_ss + kD) * 2));
+  int goff[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    koff[i] = (int)((ld_row + 16 * i) * p.k_ss * 2) + ld_chunk * 16;
-    voff[i] = (int)((ld_row * 4 + i) * p.v_ss * 2) + ld_chunk * 16;
-  }
-  const int k_tile_bytes = (int)(kBN * p.k_ss * 2);
-  const int v_tile_bytes = (int)(kBN * p.v_ss * 2);
-  u32x4 kreg[4], vreg[4];
+  for (int i = 0; i < 4; ++i)
+    goff[i] = (int)((group_b ? ld_row * 4 + i : ld_row + 16 * i) * g_ss * 2) + ld_chunk * 16;
+  const int tile_bytes = (int)(kBN * g_ss * 2);
+  u32x4 greg[4];
 
-  auto load_k = [&](int t) {
+  auto load_tile = [&](int t) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) kreg[i] = __builtin_amdgcn_raw_buffer_load_b128(krs, koff[i], t * k_tile_bytes, 0);
-  };
-  auto load_v = [&](int t) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) vreg[i] = __builtin_amdgcn_raw_buffer_load_b128(vrs, voff[i], t * v_tile_bytes, 0);
+    for (int i = 0; i < 4; ++i) greg[i] = __builtin_amdgcn_raw_buffer_load_b128(grs, goff[i], t * tile_bytes, 0);
   };
 
   // LDS position of key quad (4 consecutive keys) inside a V^T row: MFMA k-step = quad / 4,
@@ -129,26 +147,27 @@ __global__ __launch_bounds__(NW * 64, 2) void attn_fwd_bf16_d128(const FwdParams
   // and the 32 lanes of one read (rows 32 db + 0..31) then both spread over all banks.
   const int vt_xor = ((ld_chunk >> 3) & 1) | (((ld_chunk >> 2) & 1) << 1) | (((ld_chunk >> 1) & 1) << 2);
 
-  auto store_k = [&](int stage) {
-    unsigned char* ks = smem + stage * kStageBytes;
+  auto store_tile = [&](int stage) {
+    if (!group_b) {
+      unsigned char* ks = smem + stage * kStageBytes;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      *reinterpret_cast<u32x4*>(ks + (ld_row + 16 * i) * (kKStride * 2) + ld_chunk * 16) = kreg[i];
-  };
-  auto store_v = [&](int stage) {
-    unsigned char* vs = smem + stage * kStageBytes + kKBytes;
+      for (int i = 0; i < 4; ++i)
+        *reinterpret_cast<u32x4*>(ks + (ld_row + 16 * i) * (kKStride * 2) + ld_chunk * 16) = greg[i];
+    } else {
+      unsigned char* vs = smem + stage * kStageBytes + kKBytes;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      // dword j of each row holds head-dim values 2j (low half) and 2j+1 (high half)
-      u32x2 even, odd;
-      even[0] = __builtin_amdgcn_perm(vreg[1][j], vreg[0][j], 0x05040100u);
-      even[1] = __builtin_amdgcn_perm(vreg[3][j], vreg[2][j], 0x05040100u);
-      odd[0] = __builtin_amdgcn_perm(vreg[1][j], vreg[0][j], 0x07060302u);
-      odd[1] = __builtin_amdgcn_perm(vreg[3][j], vreg[2][j], 0x07060302u);
-      const int r0 = ld_chunk * 8 + ((2 * j) ^ vt_xor);
-      const int r1 = ld_chunk * 8 + ((2 * j + 1) ^ vt_xor);
-      *reinterpret_cast<u32x2*>(vs + r0 * (kVStride * 2) + vt_off) = even;
-      *reinterpret_cast<u32x2*>(vs + r1 * (kVStride * 2) + vt_off) = odd;
+      for (int j = 0; j < 4; ++j) {
+        // dword j of each row holds head-dim values 2j (low half) and 2j+1 (high half)
+        u32x2 even, odd;
+        even[0] = __builtin_amdgcn_perm(greg[1][j], greg[0][j], 0x05040100u);
+        even[1] = __builtin_amdgcn_perm(greg[3][j], greg[2][j], 0x05040100u);
+        odd[0] = __builtin_amdgcn_perm(greg[1][j], greg[0][j], 0x07060302u);
+        odd[1] = __builtin_amdgcn_perm(greg[3][j], greg[2][j], 0x07060302u);
+        const int r0 = ld_chunk * 8 + ((2 * j) ^ vt_xor);
+        const int r1 = ld_chunk * 8 + ((2 * j + 1) ^ vt_xor);
+        *reinterpret_cast<u32x2*>(vs + r0 * (kVStride * 2) + vt_off) = even;
+        *reinterpret_cast<u32x2*>(vs + r1 * (kVStride * 2) + vt_off) = odd;
+      }
     }
   };
 
@@ -161,8 +180,23 @@ __global__ __launch_bounds__(NW * 64, 2) void attn_fwd_bf16_d128(const FwdParams
   }
   const int causal_shift = p.Sc - p.Sq;
 
-  // S^T tile: 64 keys x 32 q rows per wave
-  auto qk = [&](int stage, f32x16 (&s)[2]) {
+  // ---- accumulators -----------------------------------------------------------------------------
+  f32x16 o_acc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) o_acc[i][j] = 0.f;
+  // m_ref: the score (raw, unscaled) the exponentials of this lane's Q row are taken relative to.  It
+  // follows the running maximum lazily: it only moves when the maximum has grown by more than
+  // kRescaleSlack (in log2 units of the scaled score), so exp2 arguments stay below that slack and the
+  // O accumulator is rescaled on few tiles.  The LSE does not depend on the choice of reference.
+  float m_ref = -INFINITY;
+  float l_run = 0.f;         // this lane's share of the running sum (the other 32 keys: lane ^ 32)
+  constexpr float kRescaleSlack = 8.f;
+  f32x16 s[2];               // S^T tile: 64 keys x 32 q rows per wave
+  bf16x8 pf[4];              // P^T of the current tile as bf16 B operands
+
+  auto qk = [&](int stage) {
     const unsigned char* ks = smem + stage * kStageBytes;
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
@@ -178,52 +212,51 @@ __global__ __launch_bounds__(NW * 64, 2) void attn_fwd_bf16_d128(const FwdParams
     }
   };
 
-  // ---- accumulators -----------------------------------------------------------------------------
-  f32x16 o_acc[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 16; ++j) o_acc[i][j] = 0.f;
-  // m_ref: the score (raw, unscaled) the exponentials of this lane's Q row are taken relative to.  It
-  // follows the running maximum lazily: it only moves when the maximum has grown by more than
-  // kRescaleSlack (in log2 units of the scaled score), so exp2 arguments stay below that slack and the
-  // O accumulator is rescaled on few tiles.  The LSE does not depend on the choice of reference.
-  float m_ref = -INFINITY;
-  float l_run = 0.f;         // this lane's share of the running sum (the other 32 keys: lane ^ 32)
-  constexpr float kRescaleSlack = 8.f;
-
-  f32x16 s_cur[2], s_nxt[2];
-
-  if (ntiles > 0) {
-    if (does_k) { load_k(0); store_k(0); }
-    if (does_v) { load_v(0); store_v(0); }
-    if (PIPE) {
-      if (does_k && ntiles > 1) { load_k(1); store_k(1); }
-      __syncthreads();
-      qk(0, s_cur);
-    }
-  }
-
-  for (int t = 0; t < ntiles; ++t) {
-    const int stage = t & 1;
-    if (PIPE) {
-      if (does_k && t + 2 < ntiles) load_k(t + 2);
-      if (does_v && t + 1 < ntiles) load_v(t + 1);
-    } else if (t + 1 < ntiles) {
-      if (does_k) load_k(t + 1);
-      if (does_v) load_v(t + 1);
-    }
-    __syncthreads();
+  auto pv = [&](int stage) {
     const unsigned char* vs = smem + stage * kStageBytes + kKBytes;
-
-    if (PIPE) {
-      if (t + 1 < ntiles) qk(stage ^ 1, s_nxt);
-    } else {
-      qk(stage, s_cur);
+#pragma unroll
+    for (int kstep = 0; kstep < 4; ++kstep) {
+#pragma unroll
+      for (int db = 0; db < 4; ++db) {
+        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vs + v_rd[db] + kstep * 32);
+        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kstep], o_acc[db], 0, 0, 0);
+      }
     }
+  };
 
-    // ---- mask: keys past the chunk end, and the causal diagonal ---------------------------------
+  // Matrix phase of tile t: S^T(t+1) from K stage `ks_stage` and O^T += V^T(t) P^T(t) from V stage
+  // `vs_stage`, 32 MFMAs fed by 32 LDS reads.  The reads run kFragDepth operands ahead of the MFMAs
+  // through a ring of registers, so the LDS latency is covered by the MFMAs in between.
+  auto frag_addr = [&](int i, const unsigned char* ks, const unsigned char* vs) -> const bf16x8* {
+    if (i < 16) return reinterpret_cast<const bf16x8*>(ks + k_rd + (i & 1) * (32 * kKStride * 2) + (i >> 1) * 32);
+    const int j = i - 16;
+    return reinterpret_cast<const bf16x8*>(vs + v_rd[j & 3] + (j >> 2) * 32);
+  };
+  auto matrix_phase = [&](int ks_stage, int vs_stage) {
+    const unsigned char* ks = smem + ks_stage * kStageBytes;
+    const unsigned char* vs = smem + vs_stage * kStageBytes + kKBytes;
+    bf16x8 frag[kFragDepth];
+#pragma unroll
+    for (int i = 0; i < kFragDepth; ++i) frag[i] = *frag_addr(i, ks, vs);
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      if (i < 16) {
+        const int mb = i & 1, kk = i >> 1;
+        s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag[i % kFragDepth], qf[kk], kk == 0 ? zero : s[mb], 0, 0, 0);
+      } else {
+        const int db = (i - 16) & 3, kstep = (i - 16) >> 2;
+        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag[i % kFragDepth], pf[kstep], o_acc[db], 0, 0, 0);
+      }
+      if (i + kFragDepth < 32) frag[i % kFragDepth] = *frag_addr(i + kFragDepth, ks, vs);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  // online softmax of the S^T tile of key tile t (per lane = per Q row) -> pf
+  auto softmax = [&](int t) {
     const int kv0 = t * kBN;
+    // mask: keys past the chunk end, and the causal diagonal
     bool need_mask = kv0 + kBN > p.Sc;
     if (CAUSAL) need_mask = need_mask || (kv0 + kBN - 1 > q0 + causal_shift);
     if (need_mask) {
@@ -234,16 +267,14 @@ __global__ __launch_bounds__(NW * 64, 2) void attn_fwd_bf16_d128(const FwdParams
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
           const int key = kv0 + mb * 32 + (j >> 2) * 8 + hf * 4 + (j & 3);
-          if (key > lim) s_cur[mb][j] = -INFINITY;
+          if (key > lim) s[mb][j] = -INFINITY;
         }
     }
-
-    // ---- online softmax (per lane = per Q row) ----------------------------------------------------
-    float mx = s_cur[0][0];
+    float mx = s[0][0];
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-      for (int j = 0; j < 16; ++j) mx = fmaxf(mx, s_cur[mb][j]);
+      for (int j = 0; j < 16; ++j) mx = fmaxf(mx, s[mb][j]);
     mx = pair_max(mx);
     // move the reference only when the maximum outgrew it by the slack (always on the first tile
     // that has a visible key: m_ref = -inf there)
@@ -264,45 +295,62 @@ __global__ __launch_bounds__(NW * 64, 2) void attn_fwd_bf16_d128(const FwdParams
     for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
-        const float e = fast_exp2(__builtin_fmaf(s_cur[mb][j], p.scale_log2, -msc));
-        s_cur[mb][j] = e;
+        const float e = fast_exp2(__builtin_fmaf(s[mb][j], p.scale_log2, -msc));
+        s[mb][j] = e;
         rs += e;
       }
     l_run += rs;
-
-    // ---- P^T as bf16 B operands: k-step (mb, j2) takes accumulator registers 8 j2 .. 8 j2 + 7 ---
-    bf16x8 pf[4];
+    // P^T as bf16 B operands: k-step (mb, j2) takes accumulator registers 8 j2 .. 8 j2 + 7
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
       for (int j2 = 0; j2 < 2; ++j2) {
         u32x4 w;
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          w[e] = pack_bf16(s_cur[mb][8 * j2 + 2 * e], s_cur[mb][8 * j2 + 2 * e + 1]);
+        for (int e = 0; e < 4; ++e) w[e] = pack_bf16(s[mb][8 * j2 + 2 * e], s[mb][8 * j2 + 2 * e + 1]);
         pf[mb * 2 + j2] = __builtin_bit_cast(bf16x8, w);
       }
+  };
 
-    // ---- O^T += V^T P^T ----------------------------------------------------------------------------
-#pragma unroll
-    for (int kstep = 0; kstep < 4; ++kstep) {
-#pragma unroll
-      for (int db = 0; db < 4; ++db) {
-        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vs + v_rd[db] + kstep * 32);
-        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kstep], o_acc[db], 0, 0, 0);
-      }
-    }
-
-    if (PIPE) {
-      if (does_k && t + 2 < ntiles) store_k(stage);
-      if (does_v && t + 1 < ntiles) store_v(stage ^ 1);
-#pragma unroll
-      for (int mb = 0; mb < 2; ++mb) s_cur[mb] = s_nxt[mb];
-    } else if (t + 1 < ntiles) {
-      if (does_k) store_k(stage ^ 1);
-      if (does_v) store_v(stage ^ 1);
-    }
+  // ---- prologue: tiles 0 and 1 into LDS, softmax of tile 0 ------------------------------------------
+  if (ntiles > 0) {
+    load_tile(0);
+    store_tile(0);
+    if (ntiles > 1) { load_tile(1); store_tile(1); }
+    __syncthreads();
+    qk(0);
+    softmax(0);
   }
+  // Phase p of the main loop: group A (waves 0-3) runs the matrix phase of tile p/2 on even p and its
+  // vector phase on odd p; group B does the same one phase later.  LDS stage t&1 holds K(t) / V(t);
+  // K(t+2) and V(t+2) are stored in the vector phase of tile t, after every wave has read K(t) (in the
+  // matrix phase of tile t-1) and V(t) (in the matrix phase of tile t).
+  if (kPingPong && group_b) __syncthreads();
+  for (int t = 0; t + 1 < ntiles; ++t) {
+    const int stage = t & 1;
+    // ---- matrix phase: S^T(t+1) = K(t+1) Q^T and O^T += V^T(t) P^T(t) ------------------------------
+    TR();
+    __builtin_amdgcn_s_setprio(2);
+    if (t + 2 < ntiles) load_tile(t + 2);
+    matrix_phase(stage ^ 1, stage);
+    __builtin_amdgcn_s_setprio(0);
+    TR();
+    __syncthreads();
+    TR();
+    // ---- vector phase: softmax(t+1), and this wave's share of tile t+2 into LDS ----------------------
+    softmax(t + 1);
+    TR();
+    if (t + 2 < ntiles) store_tile(stage);
+    TR();
+    __syncthreads();
+  }
+  TR();
+  if (ntiles > 0) pv((ntiles - 1) & 1);           // last tile: nothing left to prefetch or exponentiate
+  if (kPingPong && !group_b) __syncthreads();
+#ifdef MHIP_FWD_TRACE
+  __syncthreads();
+  if (blockIdx.x == 0 && p.trace) for (int i = threadIdx.x; i < 8 * 400; i += kWaves * 64) p.trace[i] = tr_buf[i];
+#endif
 
   // ---- epilogue -----------------------------------------------------------------------------------
   const float l_tot = pair_sum(l_run);
@@ -357,21 +405,17 @@ int attn_fwd_bf16(const void* q, const void* k, const void* v, void* out, float*
   p.o_sb = st[9]; p.o_ss = st[10]; p.o_sh = st[11];
   p.scale = scale;
   p.scale_log2 = scale * kLog2e;
-#ifndef MHIP_FWD_PIPE
-#define MHIP_FWD_PIPE false
-#endif
-#ifndef MHIP_FWD_WAVES
-#define MHIP_FWD_WAVES 8
-#endif
-  constexpr int kBM = MHIP_FWD_WAVES * 32;
   p.nq_tiles = (Sq + kBM - 1) / kBM;
   p.total = B * Hq * p.nq_tiles;
   p.per_xcd = (p.total + 7) / 8;
-  const dim3 grid(p.per_xcd * 8), block(MHIP_FWD_WAVES * 64);
+#ifdef MHIP_FWD_TRACE
+  { const char* e = getenv("MHIP_FWD_TRACE_PTR"); p.trace = e ? (long long*)strtoull(e, nullptr, 0) : nullptr; }
+#endif
+  const dim3 grid(p.per_xcd * 8), block(kWaves * 64);
   if (mask == MHIP_MASK_CAUSAL)
-    hipLaunchKernelGGL((attn_fwd_bf16_d128<true, MHIP_FWD_PIPE, MHIP_FWD_WAVES>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL(attn_fwd_bf16_d128<true>, grid, block, 0, stream, p);
   else
-    hipLaunchKernelGGL((attn_fwd_bf16_d128<false, MHIP_FWD_PIPE, MHIP_FWD_WAVES>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL(attn_fwd_bf16_d128<false>, grid, block, 0, stream, p);
   return launch_status();
 }
 
