@@ -20,9 +20,6 @@
 //                  0-3 and 4-7 run half a tile apart, separated by workgroup barriers, so on every
 //                  SIMD one wavefront feeds the matrix pipe while the other does exponentials.
 #include "mhip_common.hpp"
-#ifdef MHIP_FWD_TRACE
-#include <cstdlib>
-#endif
 
 namespace mhip {
 namespace {
@@ -41,7 +38,7 @@ constexpr int kOStride = kD + 8;   // epilogue staging of O, bf16 elements per r
 #define MHIP_FWD_PINGPONG 1
 #endif
 #ifndef MHIP_FWD_FRAG_DEPTH
-#define MHIP_FWD_FRAG_DEPTH 8
+#define MHIP_FWD_FRAG_DEPTH 4
 #endif
 constexpr int kFragDepth = MHIP_FWD_FRAG_DEPTH;  // LDS operand reads in flight ahead of the MFMAs
 constexpr bool kPingPong = MHIP_FWD_PINGPONG;   // 0: all wavefronts run the phases in lock step
@@ -55,9 +52,6 @@ struct FwdParams {
   int nq_tiles;      // ceil(Sq / rows per workgroup)
   int total;         // B * Hq * nq_tiles
   int per_xcd;       // ceil(total / 8)
-#ifdef MHIP_FWD_TRACE
-  long long* trace;
-#endif
 };
 
 // Buffer descriptor over `bytes` bytes at `base`: loads past the end return zero, so rows beyond the
@@ -69,13 +63,6 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
 template <bool CAUSAL>
 __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdParams p) {
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kStageBytes];
-#ifdef MHIP_FWD_TRACE
-  __shared__ long long tr_buf[8 * 400];
-  int tr_n = 0;
-#define TR() do { if (blockIdx.x == 0 && tr_n < 400) { tr_buf[(threadIdx.x >> 6) * 400 + tr_n] = clock64(); } ++tr_n; } while (0)
-#else
-#define TR() do {} while (0)
-#endif
 
   // Workgroup i runs on XCD i % 8.  Give every XCD a contiguous range of the (batch, head, q-tile)
   // order so that the workgroups sharing one K/V head also share one L2.
@@ -329,28 +316,18 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
   for (int t = 0; t + 1 < ntiles; ++t) {
     const int stage = t & 1;
     // ---- matrix phase: S^T(t+1) = K(t+1) Q^T and O^T += V^T(t) P^T(t) ------------------------------
-    TR();
     __builtin_amdgcn_s_setprio(2);
     if (t + 2 < ntiles) load_tile(t + 2);
     matrix_phase(stage ^ 1, stage);
     __builtin_amdgcn_s_setprio(0);
-    TR();
     __syncthreads();
-    TR();
     // ---- vector phase: softmax(t+1), and this wave's share of tile t+2 into LDS ----------------------
     softmax(t + 1);
-    TR();
     if (t + 2 < ntiles) store_tile(stage);
-    TR();
     __syncthreads();
   }
-  TR();
   if (ntiles > 0) pv((ntiles - 1) & 1);           // last tile: nothing left to prefetch or exponentiate
   if (kPingPong && !group_b) __syncthreads();
-#ifdef MHIP_FWD_TRACE
-  __syncthreads();
-  if (blockIdx.x == 0 && p.trace) for (int i = threadIdx.x; i < 8 * 400; i += kWaves * 64) p.trace[i] = tr_buf[i];
-#endif
 
   // ---- epilogue -----------------------------------------------------------------------------------
   const float l_tot = pair_sum(l_run);
@@ -408,9 +385,6 @@ int attn_fwd_bf16(const void* q, const void* k, const void* v, void* out, float*
   p.nq_tiles = (Sq + kBM - 1) / kBM;
   p.total = B * Hq * p.nq_tiles;
   p.per_xcd = (p.total + 7) / 8;
-#ifdef MHIP_FWD_TRACE
-  { const char* e = getenv("MHIP_FWD_TRACE_PTR"); p.trace = e ? (long long*)strtoull(e, nullptr, 0) : nullptr; }
-#endif
   const dim3 grid(p.per_xcd * 8), block(kWaves * 64);
   if (mask == MHIP_MASK_CAUSAL)
     hipLaunchKernelGGL(attn_fwd_bf16_d128<true>, grid, block, 0, stream, p);
