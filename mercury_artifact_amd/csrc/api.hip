@@ -60,15 +60,3 @@ extern "C" int mhip_attn_fwd_block(const void* q, const void* k, const void* v, 
   const int64_t strides[12] = {q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, v_sb, v_ss, v_sh, o_sb, o_ss, o_sh};
   return attn_fwd_bf16(q, k, v, out, lse, B, Sq, Sc, Hq, Hkv, strides, softmax_scale, mask, st);
 }
-
-extern "C" int64_t mhip_attn_bwd_workspace_bytes(int B, int Sq, int Sc, int Hq, int Hkv, int D) {
-  (void)B; (void)Sq; (void)Sc; (void)Hq; (void)Hkv; (void)D;
-  return 0;
-}
-
-extern "C" int mhip_attn_bwd_block(const void*, const void*, const void*, const void*, const void*,
-                                   const float*, void*, void*, void*, float*, int, int, int, int, int, int,
-                                   int64_t, int64_t, int64_t, int64_t, int64_t, int64_t,
-                                   int64_t, int64_t, int64_t, float, int, int, void*, void*) {
-  return MHIP_EUNSUPPORTED;
-}

@@ -120,42 +120,50 @@ def _(q, k, v, dropout_p, softmax_scale, causal, window_size_left, window_size_r
 
 def attn_bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_scale, causal=False,
                    deterministic=False, dq_acc: Optional[torch.Tensor] = None) -> None:
-    """Block backward through mhip_attn_bwd_block; writes dq, dk, dv in place."""
+    """Block backward through mhip_attn_bwd_block; writes every element of dq, dk, dv in place and, if
+    ``dq_acc`` (fp32, contiguous, q's shape) is given, also adds the block's dq into it."""
+    _check_block_inputs(q, k, v, 0, -1, -1, 0.0, None)
+    N.require_cuda(dout, out, softmax_lse, dq, dk, dv, dq_acc)
     B, Sq, Hq, D = q.shape
     _, Sc, Hkv, _ = k.shape
-    for name, t in (("dout", dout), ("out", out), ("dq", dq)):
-        if t.shape != q.shape or t.stride() != q.stride():
-            if t.shape != q.shape:
-                raise RuntimeError(f"{name} must have q's shape")
+    if q.dtype != torch.bfloat16:
+        raise RuntimeError("the backward kernel takes bfloat16 only")
+    for name, t, like in (("dout", dout, q), ("out", out, q), ("dq", dq, q), ("dk", dk, k), ("dv", dv, k)):
+        if t.shape != like.shape or t.dtype != torch.bfloat16:
+            raise RuntimeError(f"{name} must be bfloat16 with shape {tuple(like.shape)}")
+    if softmax_lse.shape != (B, Hq, Sq) or softmax_lse.dtype != torch.float32:
+        raise RuntimeError("softmax_lse must be float32 (B, Hq, Sq)")
+    softmax_lse = softmax_lse.contiguous()
+    if dq_acc is not None and (dq_acc.shape != q.shape or dq_acc.dtype != torch.float32
+                               or not dq_acc.is_contiguous()):
+        raise RuntimeError("dq_acc must be a contiguous float32 tensor of q's shape")
+
+    # the C ABI takes one stride triple for (q, out, dout, dq), one for (k, v), one for (dk, dv)
+    def same(*ts):
+        return all(t.stride() == ts[0].stride() and t.stride(-1) == 1 for t in ts)
+    qq, oo, dd, dq_w = (q, out, dout, dq) if same(q, out, dout, dq) else \
+        (q.contiguous(), out.contiguous(), dout.contiguous(), torch.empty_like(q, memory_format=torch.contiguous_format))
+    kk, vv = (k, v) if same(k, v) else (k.contiguous(), v.contiguous())
+    dk_w, dv_w = (dk, dv) if same(dk, dv) else \
+        (torch.empty_like(k, memory_format=torch.contiguous_format),
+         torch.empty_like(v, memory_format=torch.contiguous_format))
     lib = N.lib()
-    ws_bytes = lib.mhip_attn_bwd_workspace_bytes(B, Sq, Sc, Hq, Hkv, D)
-    ws = torch.empty((max(int(ws_bytes), 1),), dtype=torch.uint8, device=q.device)
-    doutc = dout if dout.stride() == q.stride() else dout.contiguous()
-    outc = out if out.stride() == q.stride() else out.contiguous()
-    qc = q
-    if doutc.stride() != qc.stride() or outc.stride() != qc.stride():
-        qc, doutc, outc = q.contiguous(), dout.contiguous(), out.contiguous()
-    dq_tmp = dq if dq.stride() == qc.stride() else torch.empty_like(qc)
-    if k.stride() != v.stride():
-        k, v = k.contiguous(), v.contiguous()
-    dk_tmp, dv_tmp = dk, dv
-    if dk.stride() != dv.stride():
-        dk_tmp, dv_tmp = torch.empty_like(dk, memory_format=torch.contiguous_format), \
-            torch.empty_like(dv, memory_format=torch.contiguous_format)
+    ws = torch.empty((int(lib.mhip_attn_bwd_workspace_bytes(B, Sq, Sc, Hq, Hkv, D)),), dtype=torch.uint8,
+                     device=q.device)
     with torch.cuda.device(q.device):
         code = lib.mhip_attn_bwd_block(
-            N.ptr(doutc), N.ptr(qc), N.ptr(k), N.ptr(v), N.ptr(outc), N.ptr(softmax_lse),
-            N.ptr(dq_tmp), N.ptr(dk_tmp), N.ptr(dv_tmp), N.ptr(dq_acc),
+            N.ptr(dd), N.ptr(qq), N.ptr(kk), N.ptr(vv), N.ptr(oo), N.ptr(softmax_lse),
+            N.ptr(dq_w), N.ptr(dk_w), N.ptr(dv_w), N.ptr(dq_acc),
             B, Sq, Sc, Hq, Hkv, D,
-            *_strides3(qc), *_strides3(k), *_strides3(dk_tmp),
+            *_strides3(qq), *_strides3(kk), *_strides3(dk_w),
             float(softmax_scale), N.MASK_CAUSAL if causal else N.MASK_NONE, int(bool(deterministic)),
             N.ptr(ws), N.stream_of(q))
     N.check(code, "mhip_attn_bwd_block")
-    if dq_tmp is not dq:
-        dq.copy_(dq_tmp)
-    if dk_tmp is not dk:
-        dk.copy_(dk_tmp)
-        dv.copy_(dv_tmp)
+    if dq_w is not dq:
+        dq.copy_(dq_w)
+    if dk_w is not dk:
+        dk.copy_(dk_w)
+        dv.copy_(dv_w)
 
 
 @torch.library.custom_op("mercury_amd::_flash_attn_backward", mutates_args=("dq", "dk", "dv"),
@@ -184,9 +192,6 @@ def _flash_attn_backward(
     (``torch.empty``, utils/attn_bwd_dsl.py:83-84) and every element of them is written.
     Returns ``softmax_d`` (rowsum(dout * out), (B,Hq,Sq) fp32) like flash-attn does."""
     _check_block_inputs(q, k, v, dropout_p, window_size_left, window_size_right, softcap, alibi_slopes)
-    N.require_cuda(dout, out, softmax_lse, dq, dk, dv)
-    if q.dtype != torch.bfloat16:
-        raise RuntimeError("the backward kernel takes bfloat16 only")
     attn_bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_scale, bool(causal),
                    bool(deterministic))
     return (dout.float() * out.float()).sum(-1).transpose(1, 2).contiguous()
