@@ -6,6 +6,9 @@ namespace mhip {
 int attn_fwd_bf16(const void* q, const void* k, const void* v, void* out, float* lse,
                   int B, int Sq, int Sc, int Hq, int Hkv,
                   const int64_t* strides, float scale, int mask, hipStream_t stream);
+int attn_fwd_fp8(const void* q, const void* k, const void* v, void* out, float* lse,
+                 int B, int Sq, int Sc, int Hq, int Hkv, const int64_t* strides, float scale, int mask,
+                 float q_descale, float k_descale, float v_descale, hipStream_t stream);
 }  // namespace mhip
 
 using namespace mhip;
@@ -38,7 +41,6 @@ extern "C" int mhip_attn_fwd_block(const void* q, const void* k, const void* v, 
                                    float softmax_scale, int mask, int dtype,
                                    float q_descale, float k_descale, float v_descale,
                                    void* stream) {
-  (void)q_descale; (void)k_descale; (void)v_descale;
   if (B < 0 || Sq < 0 || Sc < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return MHIP_EINVAL;
   if (!(softmax_scale > 0.f) || !(softmax_scale < INFINITY)) return MHIP_EINVAL;
   if (mask != MHIP_MASK_NONE && mask != MHIP_MASK_CAUSAL) return MHIP_EINVAL;
@@ -48,15 +50,21 @@ extern "C" int mhip_attn_fwd_block(const void* q, const void* k, const void* v, 
   if (!q || !out || !lse) return MHIP_EINVAL;
   if (Sc > 0 && (!k || !v)) return MHIP_EINVAL;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (dtype == MHIP_E4M3) return MHIP_EUNSUPPORTED;
   // 16-byte vector accesses on every row of q, k, v and out
   if (!aligned16(q) || !aligned16(out) || (Sc > 0 && (!aligned16(k) || !aligned16(v)))) return MHIP_EALIGN;
-  if (!mult8(q_sb) || !mult8(q_ss) || !mult8(q_sh) || !mult8(k_sb) || !mult8(k_ss) || !mult8(k_sh) ||
-      !mult8(v_sb) || !mult8(v_ss) || !mult8(v_sh) || !mult8(o_sb) || !mult8(o_ss) || !mult8(o_sh))
+  const bool fp8 = dtype == MHIP_E4M3;
+  auto in_ok = [fp8](int64_t x) { return fp8 ? (x & 15) == 0 : mult8(x); };     // element strides
+  if (!in_ok(q_sb) || !in_ok(q_ss) || !in_ok(q_sh) || !in_ok(k_sb) || !in_ok(k_ss) || !in_ok(k_sh) ||
+      !in_ok(v_sb) || !in_ok(v_ss) || !in_ok(v_sh) || !mult8(o_sb) || !mult8(o_ss) || !mult8(o_sh))
     return MHIP_EALIGN;
   // K / V tiles are fetched through 32-bit buffer offsets relative to the (batch, head) base
-  const int64_t kv_span = (int64_t)Sc * (k_ss > v_ss ? k_ss : v_ss) * 2;
+  const int64_t kv_span = (int64_t)Sc * (k_ss > v_ss ? k_ss : v_ss) * (fp8 ? 1 : 2);
   if (k_ss < 0 || v_ss < 0 || kv_span >= (int64_t(1) << 31)) return MHIP_EUNSUPPORTED;
   const int64_t strides[12] = {q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, v_sb, v_ss, v_sh, o_sb, o_ss, o_sh};
+  if (fp8) {
+    if (!(q_descale > 0.f) || !(k_descale > 0.f) || !(v_descale > 0.f)) return MHIP_EINVAL;
+    return attn_fwd_fp8(q, k, v, out, lse, B, Sq, Sc, Hq, Hkv, strides, softmax_scale, mask,
+                        q_descale, k_descale, v_descale, st);
+  }
   return attn_fwd_bf16(q, k, v, out, lse, B, Sq, Sc, Hq, Hkv, strides, softmax_scale, mask, st);
 }

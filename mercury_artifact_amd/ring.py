@@ -196,8 +196,9 @@ def zigzag_causal_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=True
 
 def quantize_e4m3(x: torch.Tensor):
     """Per-tensor e4m3 quantisation: scale s = amax / 448 (fp32), x_q = round-to-nearest-even(x / s)."""
-    amax = x.abs().amax().to(torch.float32)
-    scale = torch.where(amax > 0, amax / 448.0, torch.ones_like(amax))
+    amax = x.abs().amax().to(torch.float32) if x.numel() else torch.zeros((), dtype=torch.float32, device=x.device)
+    # amax / 448 in fp64, rounded once to fp32: the same bits on the host and on the device
+    scale = torch.where(amax > 0, (amax.double() / 448.0).float(), torch.ones_like(amax))
     xq = (x.to(torch.float32) / scale).clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
     return xq, scale
 

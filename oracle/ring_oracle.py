@@ -247,8 +247,9 @@ def zigzag_step(rank: int, step: int, world: int) -> Tuple[str, int]:
 # fp8 (not in the reference): per-tensor scale amax/448, round-to-nearest-even e4m3
 # --------------------------------------------------------------------------------------
 def quantize_e4m3(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
-    amax = x.abs().max().to(torch.float32)
-    scale = torch.where(amax > 0, amax / E4M3_MAX, torch.ones_like(amax))
+    amax = x.abs().max().to(torch.float32) if x.numel() else torch.zeros((), dtype=torch.float32)
+    # amax / 448 in fp64, rounded once to fp32: the same bits on the host and on the device
+    scale = torch.where(amax > 0, (amax.double() / 448.0).float(), torch.ones_like(amax))
     xq = (x.to(torch.float32) / scale).clamp(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn)
     return xq, scale
 

@@ -1,0 +1,106 @@
+"""fp8 (e4m3) forward kernel and the double-ring driver on e4m3 inputs against the CPU oracle.
+
+Two oracles on the same seeded inputs:
+  A  fp32 attention on the DE-QUANTISED tensors: isolates the kernel's own error (fp8 P, fp32 softmax):
+     |out - ref| <= 3e-2 + 2^-4 |ref| per element (2^-4 is the half-ulp of an e4m3 probability, which shows
+     undamped in rows that see one or two keys), rel-L2(out) <= 6e-2, LSE relative error <= 1e-3;
+  B  fp32 attention on the original N(0,1) tensors: the bar BASELINE.json states, max-abs(out) <= 6e-2.
+     That bar is quoted for 131072 keys; rounding V to e4m3 alone moves a single value by up to 6 %, so with
+     a few dozen keys no fp8 path can meet it.  B is therefore asserted from 1000 keys up and A everywhere.
+"""
+import pytest
+import torch
+
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _quantised(B, Sq, Sc, Hq, Hkv, seed, D=128):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, Sq, Hq, D, generator=g)
+    k = torch.randn(B, Sc, Hkv, D, generator=g)
+    v = torch.randn(B, Sc, Hkv, D, generator=g)
+    (qq, sq), (kq, sk), (vq, sv) = O.quantize_e4m3(q), O.quantize_e4m3(k), O.quantize_e4m3(v)
+    return (q, k, v), (qq, kq, vq), (sq, sk, sv)
+
+
+def _check(out, lse, ref_a, ref_b, tag, check_b=True):
+    out, lse = out.float().cpu(), lse.cpu()
+    (oa, la), (ob, _) = ref_a, ref_b
+    assert not torch.isnan(out).any(), tag
+    assert torch.equal(torch.isinf(lse), torch.isinf(la)), tag
+    excess = ((out - oa).abs() - (3e-2 + 2 ** -4 * oa.abs())).max().item()
+    assert excess <= 0, (tag, excess)
+    if oa.norm().item() > 0:
+        assert (out - oa).norm().item() / oa.norm().item() <= 6e-2, (tag, (out - oa).norm().item() / oa.norm().item())
+    else:
+        assert out.abs().max().item() == 0, tag
+    fin = ~torch.isinf(la)
+    if fin.any():
+        assert ((lse[fin] - la[fin]).abs() / la[fin].abs().clamp_min(1.0)).max().item() <= 1e-3, tag
+    if check_b:
+        assert (out - ob).abs().max().item() <= 6e-2, (tag, (out - ob).abs().max().item())
+
+
+@pytest.mark.parametrize("B,Sq,Sc,Hq,Hkv,causal", [
+    (1, 128, 128, 1, 1, False), (1, 256, 384, 2, 2, False), (2, 100, 77, 2, 1, False), (1, 300, 1000, 4, 2, False),
+    (1, 256, 256, 2, 2, True), (1, 200, 330, 2, 1, True), (1, 130, 0, 1, 1, False),
+])
+def test_fp8_block_matches_oracle(B, Sq, Sc, Hq, Hkv, causal):
+    import mercury_artifact_amd as M
+
+    print(f"fp8 case B{B} Sq{Sq} Sc{Sc} Hq{Hq} Hkv{Hkv} causal={causal}", flush=True)
+    (q, k, v), (qq, kq, vq), (sq, sk, sv) = _quantised(B, Sq, Sc, Hq, Hkv, seed=Sq + Sc)
+    scale = 128 ** -0.5
+    ref_a = O.block_attention(O.dequantize(qq, sq), O.dequantize(kq, sk), O.dequantize(vq, sv), scale, causal=causal)
+    ref_b = O.block_attention(q, k, v, scale, causal=causal)
+    out, lse, _, _ = M._flash_attn_forward(
+        q=qq.cuda(), k=kq.cuda(), v=vq.cuda(), dropout_p=0, softmax_scale=scale, causal=causal,
+        window_size_left=-1, window_size_right=-1, softcap=0.0, alibi_slopes=None, return_softmax=False,
+        q_descale=sq.cuda(), k_descale=sk.cuda(), v_descale=sv.cuda())
+    torch.cuda.synchronize()
+    assert out.dtype == torch.bfloat16 and lse.dtype == torch.float32
+    _check(out, lse, ref_a, ref_b, "fp8 block", check_b=Sc >= 1000)
+
+
+def test_fp8_product_quantiser_bits():
+    import mercury_artifact_amd as M
+
+    x = torch.randn(4, 300, 3, 128)
+    a, sa = M.quantize_e4m3(x.cuda())
+    b, sb = O.quantize_e4m3(x)
+    assert float(sa) == float(sb)
+    # the division x / s may round differently on the device in the last place, which flips a code only for
+    # values that sit on a rounding boundary: such flips are rare and move to the adjacent e4m3 code
+    ca, cb = a.cpu().view(torch.uint8).to(torch.int16), b.view(torch.uint8).to(torch.int16)
+    diff = (ca - cb).abs()
+    assert diff.max().item() <= 1 and (diff != 0).float().mean().item() <= 1e-3
+
+
+@pytest.mark.parametrize("rank", [0, 5])
+def test_fp8_double_ring(rank):
+    """BASELINE configs[4] scaled down: 2 x 4 double ring, per-tensor scales amax/448, non-causal."""
+    import mercury_artifact_amd as M
+
+    B, S, H, D, W = 1, 4096, 4, 128, 8
+    g = torch.Generator().manual_seed(7)
+    q = torch.randn(B, S, H, D, generator=g)
+    k = torch.randn(B, S, H, D, generator=g)
+    v = torch.randn(B, S, H, D, generator=g)
+    (qq, sq), (kq, sk), (vq, sv) = O.quantize_e4m3(q), O.quantize_e4m3(k), O.quantize_e4m3(v)
+    Sc = S // W
+    scale = D ** -0.5
+    order = O.double_ring_order(rank, 4, 2)
+    qs = slice(rank * Sc, (rank + 1) * Sc)
+    kvs_deq = [torch.stack([O.dequantize(kq[:, c * Sc:(c + 1) * Sc], sk), O.dequantize(vq[:, c * Sc:(c + 1) * Sc], sv)])
+               for c in range(W)]
+    ref_a = O.ring_forward(O.dequantize(qq[:, qs], sq), kvs_deq, order, scale)
+    ref_b = O.single_pass_attention(q[:, qs], k, v, scale)
+    dev = [torch.stack([kq[:, c * Sc:(c + 1) * Sc], vq[:, c * Sc:(c + 1) * Sc]]).cuda() for c in range(W)]
+    o = torch.empty(B, Sc, H, D, dtype=torch.bfloat16, device="cuda")
+    lse = torch.empty(B, H, Sc, dtype=torch.float32, device="cuda")
+    M.fp8_pack_split_kv(qq[:, qs].cuda(), dev[rank], o, lse, scale, sq.cuda(), sk.cuda(), sv.cuda(),
+                        ring=M.LocalRing((4, 2), rank, dev))
+    torch.cuda.synchronize()
+    _check(o, lse, ref_a, ref_b, "fp8 double ring")
