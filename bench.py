@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Headline benchmark: one rank's bf16 ring-attention forward step on one MI355X.
 
-Workload = BASELINE.json configs[1]: batch 1, 32 heads, head dim 128, local Q of 4096 rows, 8 KV chunks
+Workload = the headline bf16 configuration: batch 1, 32 heads, head dim 128, local Q of 4096 rows, 8 KV chunks
 of 4096 rows (32768 keys), non-causal, N(0,1) inputs cast to bf16, softmax scale 128^-0.5.
 A step = 8 block-forward kernels + the first-call cast + 7 LSE merges + the bf16 / (B,H,S) epilogue,
 driven through the same operators Mercury's generated code calls.  Inputs are resident in HBM before
@@ -20,6 +20,10 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, each counter scaled
+# by its reading for the calibration launch at the end of main() (profiles/ring_step_config1_hbm_traffic.md)
+TRAFFIC_FWD_BYTES = 134.9e6
+TRAFFIC_MERGE_BYTES = 173.2e6
 
 
 def cpu_baseline(sample_heads: int, B: int, Sq: int, D: int, W: int):
@@ -48,7 +52,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--cpu-heads", type=int, default=4, help="heads in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--cpu-heads", type=int, default=32, help="heads in the CPU baseline sample (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one rank's step on ONE GPU (the ring is emulated by local buffer rotation); "
@@ -131,6 +135,13 @@ def main() -> int:
     torch.cuda.synchronize()
     fused_ms = (time.perf_counter() - t0) / args.steps * 1e3
 
+    # one plain streaming kernel of known size (reads 128 MiB of bf16, writes 256 MiB of fp32): the
+    # calibration point for the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this script
+    calib = torch.empty(64 * 1024 * 1024, dtype=torch.bfloat16, device=dev).normal_()
+    MG.grad_accumulate(None, calib)
+    torch.cuda.synchronize()
+    del calib
+
     props = torch.cuda.get_device_properties(0)
     result = {
         "metric": "per-rank ring-attn step TFLOP/s + % MFMA peak (bf16, d128, Q 4096 x 8 chunks)",
@@ -145,17 +156,17 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": "BASELINE configs[1]: bf16 non-causal MHA, B1 H32 D128, local Q 4096 x 8 KV chunks "
+        "config": {"workload": "headline bf16 configuration: non-causal MHA, B1 H32 D128, local Q 4096 x 8 KV chunks "
                                "of 4096 (single ring, rank 0), 8 block forwards + 7 LSE merges + epilogue",
                    "flops_per_step": flops_per_step, "pct_of_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
                    "fused_epilogue_ms_per_step": round(fused_ms, 4),
                    "device": props.gcnArchName, "cus": props.multi_processor_count},
         "roofline": {"bound": "mfma", "kernel": "attn_fwd_bf16_d128", "achieved": round(fwd_tflops, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(fwd_tflops / PEAK_BF16_TFLOPS, 4),
-                     "traffic": None, "avg_launch_ms": round(fwd_ms, 4), "launches": len(fwd_events)},
+                     "traffic": TRAFFIC_FWD_BYTES, "avg_launch_ms": round(fwd_ms, 4), "launches": len(fwd_events)},
         "roofline_merge": {"bound": "hbm", "kernel": "lse_merge_kernel", "achieved": round(merge_gbs, 1),
                            "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(merge_gbs / PEAK_HBM_GBS, 4),
-                           "traffic": None, "avg_launch_ms": round(merge_ms, 5), "launches": len(real_merges),
+                           "traffic": TRAFFIC_MERGE_BYTES, "avg_launch_ms": round(merge_ms, 5), "launches": len(real_merges),
                            "bytes_per_launch": merge_bytes},
     }
     if args.cpu_heads > 0:

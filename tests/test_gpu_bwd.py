@@ -131,7 +131,7 @@ def test_bwd_ring_step():
 
 
 def test_bwd_full_size_chunk_properties():
-    """BASELINE configs[3] shape for one chunk (B1 H32 D128, Q 4096 x 4096 keys): checked on three heads
+    """The full-size backward shape for one chunk (B1 H32 D128, Q 4096 x 4096 keys): checked on three heads
     against the oracle, and by linearity in dout on all heads: bwd(2 dout) == 2 bwd(dout) up to bf16 rounding."""
     import mercury_artifact_amd as M
 

@@ -4,7 +4,7 @@ Two oracles on the same seeded inputs:
   A  fp32 attention on the DE-QUANTISED tensors: isolates the kernel's own error (fp8 P, fp32 softmax):
      |out - ref| <= 3e-2 + 2^-4 |ref| per element (2^-4 is the half-ulp of an e4m3 probability, which shows
      undamped in rows that see one or two keys), rel-L2(out) <= 6e-2, LSE relative error <= 1e-3;
-  B  fp32 attention on the original N(0,1) tensors: the bar BASELINE.json states, max-abs(out) <= 6e-2.
+  B  fp32 attention on the original N(0,1) tensors: the stated bar for fp8, max-abs(out) <= 6e-2.
      That bar is quoted for 131072 keys; rounding V to e4m3 alone moves a single value by up to 6 %, so with
      a few dozen keys no fp8 path can meet it.  B is therefore asserted from 1000 keys up and A everywhere.
 """
@@ -80,7 +80,7 @@ def test_fp8_product_quantiser_bits():
 
 @pytest.mark.parametrize("rank", [0, 5])
 def test_fp8_double_ring(rank):
-    """BASELINE configs[4] scaled down: 2 x 4 double ring, per-tensor scales amax/448, non-causal."""
+    """The fp8 double-ring configuration scaled down: 2 x 4 double ring, per-tensor scales amax/448, non-causal."""
     import mercury_artifact_amd as M
 
     B, S, H, D, W = 1, 4096, 4, 128, 8

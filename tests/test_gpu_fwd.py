@@ -1,7 +1,7 @@
 """Block forward kernel (through the C ABI) against the CPU oracle on the same seeded inputs.
 
 Tolerances (bf16 inputs, fp32 oracle on the very same bf16 values):
-  max-abs(out) <= 2e-2 and LSE relative error <= 1e-3   -- the bar BASELINE.json states;
+  max-abs(out) <= 2e-2 and LSE relative error <= 1e-3   -- the stated bar for bf16;
   rel-L2(out)  <= 1e-2                                  -- own, tighter gate (N(0,1) data gives
                                                             |out| ~ 0.1, so max-abs alone is weak).
 """
@@ -135,7 +135,7 @@ def test_fwd_rejects_what_it_does_not_implement():
 
 
 def test_fwd_chunks_merge_to_single_pass_full_size():
-    """BASELINE configs[1] at full size, checked through size-independent properties: the 8 merged
+    """The headline configuration (B1 H32 D128, Q 4096 x 8 chunks of 4096) at full size, checked through size-independent properties: the 8 merged
     chunk results equal one pass over all 32768 keys done by the same kernel (merge identity), and
     three heads are compared with the fp32 oracle."""
     import mercury_artifact_amd as M

@@ -115,7 +115,7 @@ def test_packed_reduce_ring():
 
 @pytest.mark.parametrize("rank", [0, 1, 3])
 def test_zigzag_causal_ring(rank):
-    """Causal GQA in the zigzag layout, scaled-down BASELINE configs[2] (B2 Hq32/Hkv8 D128)."""
+    """Causal GQA in the zigzag layout, a scaled-down Llama-3-8B shape (B2, Hq/Hkv = 4, D128)."""
     import mercury_artifact_amd as M
 
     B, Hq, Hkv, D, W, block = 2, 8, 2, 128, 4, 192

@@ -140,7 +140,7 @@ def test_flash_reduce_matches_update_on_packed():
 
 
 def test_config0_chunks_merge_to_single_pass():
-    """BASELINE configs[0]: fp32, B1 H4 D64, Q 1024, K/V 1024 in 4 chunks of 256, seed 0."""
+    """The CPU plumbing configuration: fp32, B1 H4 D64, Q 1024, K/V 1024 in 4 chunks of 256, seed 0."""
     torch.manual_seed(0)
     q, k, v = (torch.randn(1, 1024, 4, 64) for _ in range(3))
     scale = 64 ** -0.5
