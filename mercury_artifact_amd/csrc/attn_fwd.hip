@@ -211,6 +211,88 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     }
   };
 
+  // ---- online softmax of one S^T tile (per lane = per Q row) -> pf, cut into pieces ---------------------
+  // The first kEarly exponentials are computed inside the matrix phase, behind the O^T MFMAs; the rest,
+  // the packing to bf16 and the (rare) rescale of O in the vector phase.  State shared by the pieces:
+  float mx = -INFINITY, msc = 0.f, rs = 0.f, alpha = 1.f;
+  // keys past the chunk end and the causal diagonal -> -inf
+  auto sm_mask = [&](int t) {
+    const int kv0 = t * kBN;
+    bool need_mask = kv0 + kBN > p.Sc;
+    if (CAUSAL) need_mask = need_mask || (kv0 + kBN - 1 > q0 + causal_shift);
+    if (need_mask) {
+      int lim = p.Sc - 1;                                   // last visible key of this lane's row
+      if (CAUSAL) { const int c = my_q + causal_shift; lim = c < lim ? c : lim; }
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const int key = kv0 + mb * 32 + (j >> 2) * 8 + hf * 4 + (j & 3);
+          if (key > lim) s[mb][j] = -INFINITY;
+        }
+    }
+  };
+  // running maximum over accumulator registers 8i .. 8i+7 (i = 0..3)
+  auto sm_max = [&](int i) {
+    const int mb = i >> 1, base = (i & 1) * 8;
+    if (i == 0) mx = s[0][0];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) mx = fmaxf(mx, s[mb][base + j]);
+  };
+  // Combine with the other 32 keys and move the reference when the maximum outgrew it by the slack
+  // (always on the first tile with a visible key: m_ref = -inf there).  The factor alpha that O and the
+  // running sum owe to the move is applied later, by sm_finish, once the MFMAs of the tile before have
+  // landed in O.
+  auto sm_reference = [&]() {
+    mx = pair_max(mx);
+    const bool grow = (mx - m_ref) * p.scale_log2 > kRescaleSlack;     // false for NaN (-inf - -inf)
+    const float m_new = grow ? mx : m_ref;
+    alpha = (grow && m_new != -INFINITY) ? fast_exp2((m_ref - m_new) * p.scale_log2) : 1.f;
+    m_ref = m_new;
+    msc = (m_ref == -INFINITY) ? 0.f : m_ref * p.scale_log2;
+    rs = 0.f;
+  };
+  // exponentials of accumulator registers 2e, 2e+1 (e = 0..15, counted over both 32-key blocks)
+  auto sm_exp = [&](int e) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int j = 2 * e + u;
+      const float x = fast_exp2(__builtin_fmaf(s[j >> 4][j & 15], p.scale_log2, -msc));
+      s[j >> 4][j & 15] = x;
+      rs += x;
+    }
+  };
+  // rescale (only if some row of the wave moved its reference), running sum, P^T as bf16 B operands:
+  // k-step (mb, j2) takes accumulator registers 8 j2 .. 8 j2 + 7
+  auto sm_finish = [&]() {
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) o_acc[db][j] *= alpha;
+    }
+    l_run = l_run * alpha + rs;
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int j2 = 0; j2 < 2; ++j2) {
+        u32x4 w;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = pack_bf16(s[mb][8 * j2 + 2 * e], s[mb][8 * j2 + 2 * e + 1]);
+        pf[mb * 2 + j2] = __builtin_bit_cast(bf16x8, w);
+      }
+  };
+  constexpr int kEarly = 10;     // pairs of exponentials done in the matrix phase (slots 22..31)
+  auto softmax_all = [&](int t) {
+    sm_mask(t);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sm_max(i);
+    sm_reference();
+#pragma unroll
+    for (int e = 0; e < 16; ++e) sm_exp(e);
+    sm_finish();
+  };
+
   // Matrix phase of tile t: S^T(t+1) from K stage `ks_stage` and O^T += V^T(t) P^T(t) from V stage
   // `vs_stage`, 32 MFMAs fed by 32 LDS reads.  The reads run kFragDepth operands ahead of the MFMAs
   // through a ring of registers, so the LDS latency is covered by the MFMAs in between.
@@ -219,7 +301,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     const int j = i - 16;
     return reinterpret_cast<const bf16x8*>(vs + v_rd[j & 3] + (j >> 2) * 32);
   };
-  auto matrix_phase = [&](int ks_stage, int vs_stage) {
+  auto matrix_phase = [&](int t_next, int ks_stage, int vs_stage) {
     const unsigned char* ks = smem + ks_stage * kStageBytes;
     const unsigned char* vs = smem + vs_stage * kStageBytes + kKBytes;
     bf16x8 frag[kFragDepth];
@@ -236,67 +318,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
         o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag[i % kFragDepth], pf[kstep], o_acc[db], 0, 0, 0);
       }
       if (i + kFragDepth < 32) frag[i % kFragDepth] = *frag_addr(i + kFragDepth, ks, vs);
+      // S^T(t_next) is complete after slot 15; its softmax starts here, in the shadow of the O^T MFMAs
+      if (i == 16) sm_mask(t_next);
+      if (i >= 17 && i < 21) sm_max(i - 17);
+      if (i == 21) sm_reference();
+      if (i >= 22) sm_exp(i - 22);
       __builtin_amdgcn_sched_barrier(0);
     }
-  };
-
-  // online softmax of the S^T tile of key tile t (per lane = per Q row) -> pf
-  auto softmax = [&](int t) {
-    const int kv0 = t * kBN;
-    // mask: keys past the chunk end, and the causal diagonal
-    bool need_mask = kv0 + kBN > p.Sc;
-    if (CAUSAL) need_mask = need_mask || (kv0 + kBN - 1 > q0 + causal_shift);
-    if (need_mask) {
-      int lim = p.Sc - 1;                                   // last visible key of this lane's row
-      if (CAUSAL) { const int c = my_q + causal_shift; lim = c < lim ? c : lim; }
-#pragma unroll
-      for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-          const int key = kv0 + mb * 32 + (j >> 2) * 8 + hf * 4 + (j & 3);
-          if (key > lim) s[mb][j] = -INFINITY;
-        }
-    }
-    float mx = s[0][0];
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-      for (int j = 0; j < 16; ++j) mx = fmaxf(mx, s[mb][j]);
-    mx = pair_max(mx);
-    // move the reference only when the maximum outgrew it by the slack (always on the first tile
-    // that has a visible key: m_ref = -inf there)
-    const bool grow = (mx - m_ref) * p.scale_log2 > kRescaleSlack;     // false for NaN (-inf - -inf)
-    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-      const float m_new = grow ? mx : m_ref;
-      const float alpha = (m_new == -INFINITY) ? 1.f : fast_exp2((m_ref - m_new) * p.scale_log2);
-      m_ref = m_new;
-      l_run *= alpha;
-#pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) o_acc[db][j] *= alpha;
-    }
-    const float msc = (m_ref == -INFINITY) ? 0.f : m_ref * p.scale_log2;
-    float rs = 0.f;
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const float e = fast_exp2(__builtin_fmaf(s[mb][j], p.scale_log2, -msc));
-        s[mb][j] = e;
-        rs += e;
-      }
-    l_run += rs;
-    // P^T as bf16 B operands: k-step (mb, j2) takes accumulator registers 8 j2 .. 8 j2 + 7
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-      for (int j2 = 0; j2 < 2; ++j2) {
-        u32x4 w;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) w[e] = pack_bf16(s[mb][8 * j2 + 2 * e], s[mb][8 * j2 + 2 * e + 1]);
-        pf[mb * 2 + j2] = __builtin_bit_cast(bf16x8, w);
-      }
   };
 
   // ---- prologue: tiles 0 and 1 into LDS, softmax of tile 0 ------------------------------------------
@@ -306,7 +334,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     if (ntiles > 1) { load_tile(1); store_tile(1); }
     __syncthreads();
     qk(0);
-    softmax(0);
+    softmax_all(0);
   }
   // Phase p of the main loop: group A (waves 0-3) runs the matrix phase of tile p/2 on even p and its
   // vector phase on odd p; group B does the same one phase later.  LDS stage t&1 holds K(t) / V(t);
@@ -318,11 +346,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     // ---- matrix phase: S^T(t+1) = K(t+1) Q^T and O^T += V^T(t) P^T(t) ------------------------------
     __builtin_amdgcn_s_setprio(2);
     if (t + 2 < ntiles) load_tile(t + 2);
-    matrix_phase(stage ^ 1, stage);
+    matrix_phase(t + 1, stage ^ 1, stage);
     __builtin_amdgcn_s_setprio(0);
     __syncthreads();
     // ---- vector phase: softmax(t+1), and this wave's share of tile t+2 into LDS ----------------------
-    softmax(t + 1);
+#pragma unroll
+    for (int e = kEarly; e < 16; ++e) sm_exp(e);
+    sm_finish();
     if (t + 2 < ntiles) store_tile(stage);
     __syncthreads();
   }
