@@ -32,7 +32,9 @@ constexpr int kKStride = kD + 8;   // bf16 elements per K row in LDS (272 B: 16 
 constexpr int kVStride = kBN + 8;  // bf16 elements per V^T row in LDS (144 B)
 constexpr int kKBytes = kBN * kKStride * 2;   // 17408
 constexpr int kVBytes = kD * kVStride * 2;    // 18432
-constexpr int kStageBytes = kKBytes + kVBytes;
+constexpr int kKStages = 3;         // K(t+1) .. K(t+3) live while tile t is processed
+constexpr int kVStages = 2;
+constexpr int kVBase = kKStages * kKBytes;
 constexpr int kOStride = kD + 8;   // epilogue staging of O, bf16 elements per row
 #ifndef MHIP_FWD_PINGPONG
 #define MHIP_FWD_PINGPONG 1
@@ -62,7 +64,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
 
 template <bool CAUSAL>
 __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdParams p) {
-  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kStageBytes];
+  __shared__ __attribute__((aligned(16))) unsigned char smem[kKStages * kKBytes + kVStages * kVBytes];
 
   // Workgroup i runs on XCD i % 8.  Give every XCD a contiguous range of the (batch, head, q-tile)
   // order so that the workgroups sharing one K/V head also share one L2.
@@ -120,7 +122,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
   for (int i = 0; i < 4; ++i)
     goff[i] = (int)((group_b ? ld_row * 4 + i : ld_row + 16 * i) * g_ss * 2) + ld_chunk * 16;
   const int tile_bytes = (int)(kBN * g_ss * 2);
-  u32x4 greg[4];
+  u32x4 greg[4];   // staging registers: a tile's loads are issued a whole tile before their LDS stores
 
   auto load_tile = [&](int t) {
 #pragma unroll
@@ -136,12 +138,12 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
 
   auto store_tile = [&](int stage) {
     if (!group_b) {
-      unsigned char* ks = smem + stage * kStageBytes;
+      unsigned char* ks = smem + stage * kKBytes;
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         *reinterpret_cast<u32x4*>(ks + (ld_row + 16 * i) * (kKStride * 2) + ld_chunk * 16) = greg[i];
     } else {
-      unsigned char* vs = smem + stage * kStageBytes + kKBytes;
+      unsigned char* vs = smem + kVBase + stage * kVBytes;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         // dword j of each row holds head-dim values 2j (low half) and 2j+1 (high half)
@@ -184,7 +186,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
   bf16x8 pf[4];              // P^T of the current tile as bf16 B operands
 
   auto qk = [&](int stage) {
-    const unsigned char* ks = smem + stage * kStageBytes;
+    const unsigned char* ks = smem + stage * kKBytes;
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
@@ -200,7 +202,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
   };
 
   auto pv = [&](int stage) {
-    const unsigned char* vs = smem + stage * kStageBytes + kKBytes;
+    const unsigned char* vs = smem + kVBase + stage * kVBytes;
 #pragma unroll
     for (int kstep = 0; kstep < 4; ++kstep) {
 #pragma unroll
@@ -301,12 +303,17 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     const int j = i - 16;
     return reinterpret_cast<const bf16x8*>(vs + v_rd[j & 3] + (j >> 2) * 32);
   };
-  auto matrix_phase = [&](int t_next, int ks_stage, int vs_stage) {
-    const unsigned char* ks = smem + ks_stage * kStageBytes;
-    const unsigned char* vs = smem + vs_stage * kStageBytes + kKBytes;
-    bf16x8 frag[kFragDepth];
+  // The first kFragDepth operands (all of K) are read before the barrier that opens the phase, by
+  // first_frags, so the matrix pipe starts without waiting for LDS.
+  bf16x8 frag[kFragDepth];
+  auto first_frags = [&](int ks_stage) {
+    const unsigned char* ks = smem + ks_stage * kKBytes;
 #pragma unroll
-    for (int i = 0; i < kFragDepth; ++i) frag[i] = *frag_addr(i, ks, vs);
+    for (int i = 0; i < kFragDepth; ++i) frag[i] = *frag_addr(i, ks, ks);
+  };
+  auto matrix_phase = [&](int t_next, int ks_stage, int vs_stage) {
+    const unsigned char* ks = smem + ks_stage * kKBytes;
+    const unsigned char* vs = smem + kVBase + vs_stage * kVBytes;
     const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
@@ -327,36 +334,45 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     }
   };
 
-  // ---- prologue: tiles 0 and 1 into LDS, softmax of tile 0 ------------------------------------------
+  // ---- prologue: the first tiles into LDS, softmax of tile 0 -------------------------------------------
+  // K is staged three tiles ahead and V two: K(t+2) must be readable one phase before the matrix phase
+  // that consumes it, for first_frags.
+  const int lead = group_b ? kVStages : kKStages;
   if (ntiles > 0) {
     load_tile(0);
     store_tile(0);
     if (ntiles > 1) { load_tile(1); store_tile(1); }
+    if (!group_b && ntiles > 2) { load_tile(2); store_tile(2); }
+    if (lead < ntiles) load_tile(lead);   // lands during the first tile, stored in its vector phase
     __syncthreads();
     qk(0);
     softmax_all(0);
+    if (ntiles > 1) first_frags(1);
   }
   // Phase p of the main loop: group A (waves 0-3) runs the matrix phase of tile p/2 on even p and its
-  // vector phase on odd p; group B does the same one phase later.  LDS stage t&1 holds K(t) / V(t);
-  // K(t+2) and V(t+2) are stored in the vector phase of tile t, after every wave has read K(t) (in the
-  // matrix phase of tile t-1) and V(t) (in the matrix phase of tile t).
+  // vector phase on odd p; group B does the same one phase later.  K(t) lives in K stage t % 3, V(t) in V
+  // stage t & 1.  The vector phase of tile t stores K(t+3) over K(t) and V(t+2) over V(t): every wave has
+  // read K(t) in the matrix phase of tile t-1 and V(t) in the matrix phase of tile t.
   if (kPingPong && group_b) __syncthreads();
+  int k3 = 0;   // t % 3
   for (int t = 0; t + 1 < ntiles; ++t) {
-    const int stage = t & 1;
-    // ---- matrix phase: S^T(t+1) = K(t+1) Q^T and O^T += V^T(t) P^T(t) ------------------------------
+    const int k3n = k3 == 2 ? 0 : k3 + 1;          // (t+1) % 3
+    // ---- matrix phase: S^T(t+1) = K(t+1) Q^T and O^T += V^T(t) P^T(t), first part of softmax(t+1) ------
     __builtin_amdgcn_s_setprio(2);
-    if (t + 2 < ntiles) load_tile(t + 2);
-    matrix_phase(t + 1, stage ^ 1, stage);
+    matrix_phase(t + 1, k3n, t & 1);
     __builtin_amdgcn_s_setprio(0);
     __syncthreads();
-    // ---- vector phase: softmax(t+1), and this wave's share of tile t+2 into LDS ----------------------
+    // ---- vector phase: rest of softmax(t+1), this wave's share of the next tiles into LDS ------------------
 #pragma unroll
     for (int e = kEarly; e < 16; ++e) sm_exp(e);
     sm_finish();
-    if (t + 2 < ntiles) store_tile(stage);
+    if (t + lead < ntiles) store_tile(group_b ? (t & 1) : k3);   // loaded a tile ago
+    if (t + lead + 1 < ntiles) load_tile(t + lead + 1);           // a whole tile to land
+    if (t + 2 < ntiles) first_frags(k3n == 2 ? 0 : k3n + 1);      // K(t+2), for the next matrix phase
+    k3 = k3n;
     __syncthreads();
   }
-  if (ntiles > 0) pv((ntiles - 1) & 1);           // last tile: nothing left to prefetch or exponentiate
+  if (ntiles > 0) pv((ntiles - 1) & 1);             // last tile: nothing left to prefetch or exponentiate
   if (kPingPong && !group_b) __syncthreads();
 
   // ---- epilogue -----------------------------------------------------------------------------------
