@@ -54,6 +54,7 @@ struct FwdParams {
   int nq_tiles;      // ceil(Sq / rows per workgroup)
   int total;         // B * Hq * nq_tiles
   int per_xcd;       // ceil(total / 8)
+  int heads_per_xcd; // (batch, head) pairs per XCD when they divide evenly, else 0
 };
 
 // Buffer descriptor over `bytes` bytes at `base`: loads past the end return zero, so rows beyond the
@@ -68,14 +69,28 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
 
   // Workgroup i runs on XCD i % 8.  Give every XCD a contiguous range of the (batch, head, q-tile)
   // order so that the workgroups sharing one K/V head also share one L2.
-  const int logical = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
-  if (logical >= p.total) return;
-  int qt = logical % p.nq_tiles;
-  const int bh = logical / p.nq_tiles;
+  // Under the causal mask a Q tile's work grows with its index, so there the order is longest tiles
+  // first across all heads (of the XCD when the heads divide evenly over the XCDs, of the launch
+  // otherwise): the short tiles fill the tail.
+  int qt, bh;
+  if (!CAUSAL) {
+    const int logical = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
+    if (logical >= p.total) return;
+    qt = logical % p.nq_tiles;
+    bh = logical / p.nq_tiles;
+  } else if (p.heads_per_xcd > 0) {
+    const int local = blockIdx.x >> 3;
+    qt = p.nq_tiles - 1 - local / p.heads_per_xcd;
+    bh = (blockIdx.x & 7) * p.heads_per_xcd + local % p.heads_per_xcd;
+  } else {
+    if ((int)blockIdx.x >= p.total) return;
+    const int nbh = p.B * p.Hq;
+    qt = p.nq_tiles - 1 - (int)blockIdx.x / nbh;
+    bh = (int)blockIdx.x % nbh;
+  }
   const int hq = bh % p.Hq;
   const int b = bh / p.Hq;
   const int hk = hq / p.group;
-  if (CAUSAL) qt = p.nq_tiles - 1 - qt;          // longest rows first
   const int q0 = qt * kBM;
 
   const int tid = threadIdx.x;
@@ -284,7 +299,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
         pf[mb * 2 + j2] = __builtin_bit_cast(bf16x8, w);
       }
   };
-  constexpr int kEarly = 10;     // pairs of exponentials done in the matrix phase (slots 22..31)
+#ifndef MHIP_FWD_EARLY
+#define MHIP_FWD_EARLY 10
+#endif
+  constexpr int kEarly = MHIP_FWD_EARLY;     // pairs of exponentials done in the matrix phase (slots 22..31)
   auto softmax_all = [&](int t) {
     sm_mask(t);
 #pragma unroll
@@ -329,7 +347,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
       if (i == 16) sm_mask(t_next);
       if (i >= 17 && i < 21) sm_max(i - 17);
       if (i == 21) sm_reference();
-      if (i >= 22) sm_exp(i - 22);
+      if (i >= 22 && i - 22 < kEarly) sm_exp(i - 22);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -431,6 +449,7 @@ int attn_fwd_bf16(const void* q, const void* k, const void* v, void* out, float*
   p.nq_tiles = (Sq + kBM - 1) / kBM;
   p.total = B * Hq * p.nq_tiles;
   p.per_xcd = (p.total + 7) / 8;
+  p.heads_per_xcd = (B * Hq) % 8 == 0 ? (B * Hq) / 8 : 0;
   const dim3 grid(p.per_xcd * 8), block(kWaves * 64);
   if (mask == MHIP_MASK_CAUSAL)
     hipLaunchKernelGGL(attn_fwd_bf16_d128<true>, grid, block, 0, stream, p);
