@@ -44,6 +44,7 @@ struct BwdParams {
   int n_tiles;      // stationary tiles per (batch, head)
   int total;
   int per_xcd;
+  int heads_per_xcd;   // (batch, stationary head) pairs per XCD when they divide evenly, else 0
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
@@ -79,10 +80,29 @@ template <bool DQ, bool CAUSAL>
 __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
   __shared__ __attribute__((aligned(16))) unsigned char smem[kSmemBytes];
 
-  const int logical = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
-  if (logical >= p.total) return;
-  const int st_tile = logical % p.n_tiles;
-  const int bh = logical / p.n_tiles;
+  // Workgroup i runs on XCD i % 8: every XCD gets a contiguous range of (batch, head) pairs.  Under the
+  // causal mask the work of a stationary tile grows (query tiles) or shrinks (key tiles) with its index:
+  // such launches run the longest tiles first, across all heads.
+  int st_tile, bh;
+  if (!CAUSAL) {
+    const int logical = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
+    if (logical >= p.total) return;
+    st_tile = logical % p.n_tiles;
+    bh = logical / p.n_tiles;
+  } else {
+    int rank;                                       // position in longest-first order
+    if (p.heads_per_xcd > 0) {
+      const int local = blockIdx.x >> 3;
+      rank = local / p.heads_per_xcd;
+      bh = (blockIdx.x & 7) * p.heads_per_xcd + local % p.heads_per_xcd;
+    } else {
+      if ((int)blockIdx.x >= p.total) return;
+      const int nbh = p.total / p.n_tiles;
+      rank = (int)blockIdx.x / nbh;
+      bh = (int)blockIdx.x % nbh;
+    }
+    st_tile = DQ ? p.n_tiles - 1 - rank : rank;
+  }
   const int hs = DQ ? bh % p.Hq : bh % p.Hkv;       // stationary head: a q head (DQ) or a kv head
   const int b = DQ ? bh / p.Hq : bh / p.Hkv;
   const int r0 = st_tile * kRowsPerWg;
@@ -434,6 +454,7 @@ extern "C" int mhip_attn_bwd_block(const void* dout, const void* q, const void* 
     p.n_tiles = (Sq + kRowsPerWg - 1) / kRowsPerWg;
     p.total = B * Hq * p.n_tiles;
     p.per_xcd = (p.total + 7) / 8;
+    p.heads_per_xcd = (B * Hq) % 8 == 0 ? (B * Hq) / 8 : 0;
     if (causal) hipLaunchKernelGGL((bwd_main<true, true>), dim3(p.per_xcd * 8), dim3(256), 0, st, p);
     else hipLaunchKernelGGL((bwd_main<true, false>), dim3(p.per_xcd * 8), dim3(256), 0, st, p);
   }
@@ -442,6 +463,7 @@ extern "C" int mhip_attn_bwd_block(const void* dout, const void* q, const void* 
     p.n_tiles = (Sc + kRowsPerWg - 1) / kRowsPerWg;
     p.total = B * Hkv * p.n_tiles;
     p.per_xcd = (p.total + 7) / 8;
+    p.heads_per_xcd = (B * Hkv) % 8 == 0 ? (B * Hkv) / 8 : 0;
     if (causal) hipLaunchKernelGGL((bwd_main<false, true>), dim3(p.per_xcd * 8), dim3(256), 0, st, p);
     else hipLaunchKernelGGL((bwd_main<false, false>), dim3(p.per_xcd * 8), dim3(256), 0, st, p);
   }

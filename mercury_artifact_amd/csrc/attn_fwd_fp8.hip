@@ -36,7 +36,7 @@ struct Fp8Params {
   float scale_eff;       // softmax_scale * q_descale * k_descale: natural-log scale of the integer-like dot
   float scale_log2;      // scale_eff * log2(e)
   float out_mul;         // v_descale
-  int nq_tiles, total, per_xcd;
+  int nq_tiles, total, per_xcd, heads_per_xcd;
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
@@ -51,14 +51,28 @@ template <bool CAUSAL>
 __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Params p) {
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kStageBytes];
 
-  const int logical = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
-  if (logical >= p.total) return;
-  int qt = logical % p.nq_tiles;
-  const int bh = logical / p.nq_tiles;
+  // Workgroup i runs on XCD i % 8: every XCD gets a contiguous range of (batch, head) pairs, so the
+  // workgroups that share a K/V head share an L2.  Causal launches run the longest Q tiles first,
+  // across all heads.
+  int qt, bh;
+  if (!CAUSAL) {
+    const int logical = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
+    if (logical >= p.total) return;
+    qt = logical % p.nq_tiles;
+    bh = logical / p.nq_tiles;
+  } else if (p.heads_per_xcd > 0) {
+    const int local = blockIdx.x >> 3;
+    qt = p.nq_tiles - 1 - local / p.heads_per_xcd;
+    bh = (blockIdx.x & 7) * p.heads_per_xcd + local % p.heads_per_xcd;
+  } else {
+    if ((int)blockIdx.x >= p.total) return;
+    const int nbh = p.B * p.Hq;
+    qt = p.nq_tiles - 1 - (int)blockIdx.x / nbh;
+    bh = (int)blockIdx.x % nbh;
+  }
   const int hq = bh % p.Hq;
   const int b = bh / p.Hq;
   const int hk = hq / p.group;
-  if (CAUSAL) qt = p.nq_tiles - 1 - qt;
   const int q0 = qt * kBM;
 
   const int tid = threadIdx.x;
@@ -306,6 +320,7 @@ int attn_fwd_fp8(const void* q, const void* k, const void* v, void* out, float* 
   p.nq_tiles = (Sq + kBM - 1) / kBM;
   p.total = B * Hq * p.nq_tiles;
   p.per_xcd = (p.total + 7) / 8;
+  p.heads_per_xcd = (B * Hq) % 8 == 0 ? (B * Hq) / 8 : 0;
   const dim3 grid(p.per_xcd * 8), block(kWaves * 64);
   if (mask == MHIP_MASK_CAUSAL) hipLaunchKernelGGL(attn_fwd_fp8_d128<true>, grid, block, 0, stream, p);
   else hipLaunchKernelGGL(attn_fwd_fp8_d128<false>, grid, block, 0, stream, p);
