@@ -1,0 +1,110 @@
+"""The two large configurations at full size, through size-independent properties plus oracle spot checks.
+
+  * causal GQA in the zigzag layout: B2, 32 query / 8 KV heads, D128, 8 ranks x 2 blocks of 4096 rows
+    (65536-token sequence), bf16;
+  * e4m3 forward over a 2 x 4 double ring: B1, 32 heads, D128, Q shard 16384 rows x 8 KV chunks of 16384
+    (131072-token sequence), per-tensor scales amax / 448.
+
+At these sizes the fp32 oracle cannot do the whole problem in seconds, so each test checks
+  (1) the merged ring result against ONE pass of the same block kernel over all visible keys
+      (the merge identity: folding chunk results by LSE rescaling reproduces the single softmax), and
+  (2) a few heads x 128-row windows against the CPU oracle over all their keys, to the stated tolerances
+      (bf16: max-abs(out) <= 2e-2, LSE rel <= 1e-3; fp8: max-abs(out) <= 6e-2 against fp32 attention on
+      the un-quantised values, and the tighter own bounds against attention on the de-quantised values).
+Inputs are drawn on the device from a seeded generator and copied back for the oracle.
+"""
+import pytest
+import torch
+
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def test_zigzag_causal_gqa_full_size():
+    import mercury_artifact_amd as M
+
+    B, Hq, Hkv, D, W, block = 2, 32, 8, 128, 8, 4096
+    S = 2 * W * block
+    rank = 2
+    scale = D ** -0.5
+    g = torch.Generator(device="cuda").manual_seed(11)
+    k = torch.randn(B, S, Hkv, D, generator=g, device="cuda").bfloat16()
+    v = torch.randn(B, S, Hkv, D, generator=g, device="cuda").bfloat16()
+    pos = [torch.as_tensor(O.zigzag_local_positions(r, W, block), device="cuda") for r in range(W)]
+    q_full_rows = torch.randn(B, 2 * block, Hq, D, generator=g, device="cuda").bfloat16()   # rank's Q only
+    chunks = [torch.stack([k[:, p], v[:, p]]) for p in pos]
+    o = torch.empty_like(q_full_rows)
+    lse = torch.empty(B, Hq, 2 * block, dtype=torch.float32, device="cuda")
+    print("zigzag ring step", flush=True)
+    M.zigzag_causal_pack_kv(q_full_rows, chunks[rank], o, lse, scale, ring=M.LocalRing((W,), rank, chunks))
+    torch.cuda.synchronize()
+
+    # (1) each local block against one causal pass over its whole key prefix
+    for half, blk in enumerate((rank, 2 * W - 1 - rank)):
+        rows = slice(half * block, (half + 1) * block)
+        end = (blk + 1) * block
+        print(f"single pass, block {blk}", flush=True)
+        so, sl = M.attn_fwd_block(q_full_rows[:, rows], k[:, :end], v[:, :end], scale, causal=True)
+        torch.cuda.synchronize()
+        assert (o[:, rows].float() - so.float()).abs().max().item() <= 4e-3
+        assert ((lse[:, :, rows] - sl).abs() / sl.abs().clamp_min(1.0)).max().item() <= 1e-5
+
+    # (2) oracle on 128-row windows: the first rows of the early block, the last rows of the late block
+    heads = [0, 17, 31]
+    kvh = [h // (Hq // Hkv) for h in heads]
+    for half, blk, first in ((0, rank, True), (1, 2 * W - 1 - rank, False)):
+        lo = half * block + (0 if first else block - 128)
+        gpos = blk * block + (0 if first else block - 128)          # global position of the window's first row
+        end = gpos + 128
+        qw = q_full_rows[1:2, lo:lo + 128][:, :, heads].float().cpu()
+        kw = k[1:2, :end][:, :, kvh].float().cpu()
+        vw = v[1:2, :end][:, :, kvh].float().cpu()
+        ro, rl = O.block_attention(qw, kw, vw, scale, causal=True)
+        go = o[1:2, lo:lo + 128][:, :, heads].float().cpu()
+        gl = lse[1:2, heads, lo:lo + 128].cpu()
+        assert (go - ro).abs().max().item() <= 2e-2
+        assert (go - ro).norm().item() / ro.norm().item() <= 1e-2
+        assert ((gl - rl).abs() / rl.abs().clamp_min(1.0)).max().item() <= 1e-3
+
+
+def test_fp8_double_ring_full_size():
+    import mercury_artifact_amd as M
+
+    B, H, D, W, Sc = 1, 32, 128, 8, 16384
+    S = W * Sc
+    rank = 5
+    scale = D ** -0.5
+    g = torch.Generator(device="cuda").manual_seed(12)
+    k = torch.randn(B, S, H, D, generator=g, device="cuda")
+    v = torch.randn(B, S, H, D, generator=g, device="cuda")
+    q = torch.randn(B, Sc, H, D, generator=g, device="cuda")          # this rank's shard
+    (qq, sq), (kq, sk), (vq, sv) = M.quantize_e4m3(q), M.quantize_e4m3(k), M.quantize_e4m3(v)
+    chunks = [torch.stack([kq[:, c * Sc:(c + 1) * Sc], vq[:, c * Sc:(c + 1) * Sc]]) for c in range(W)]
+    o = torch.empty(B, Sc, H, D, dtype=torch.bfloat16, device="cuda")
+    lse = torch.empty(B, H, Sc, dtype=torch.float32, device="cuda")
+    print("fp8 double ring step", flush=True)
+    M.fp8_pack_split_kv(qq, chunks[rank], o, lse, scale, sq, sk, sv, ring=M.LocalRing((4, 2), rank, chunks))
+    torch.cuda.synchronize()
+
+    # (1) one pass of the same kernel over all 131072 keys
+    print("fp8 single pass", flush=True)
+    so, sl = M.attn_fwd_block(qq, kq, vq, scale, q_descale=sq, k_descale=sk, v_descale=sv)
+    torch.cuda.synchronize()
+    assert (o.float() - so.float()).abs().max().item() <= 4e-3
+    assert ((lse - sl).abs() / sl.abs().clamp_min(1.0)).max().item() <= 1e-5
+
+    # (2) oracle on two heads x two 64-row windows, over all keys
+    heads = [3, 30]
+    rows = torch.cat([torch.arange(0, 64), torch.arange(Sc - 64, Sc)])
+    go = o[:, rows][:, :, heads].float().cpu()
+    gl = lse[:, heads][:, :, rows].cpu()
+    q_deq = O.dequantize(qq[:, rows][:, :, heads].cpu(), sq.cpu())
+    k_deq = O.dequantize(kq[:, :, heads].cpu(), sk.cpu())
+    v_deq = O.dequantize(vq[:, :, heads].cpu(), sv.cpu())
+    oa, la = O.block_attention(q_deq, k_deq, v_deq, scale)
+    ob, _ = O.block_attention(q[:, rows][:, :, heads].cpu(), k[:, :, heads].cpu(), v[:, :, heads].cpu(), scale)
+    assert ((go - oa).abs() - (3e-2 + 2 ** -4 * oa.abs())).max().item() <= 0
+    assert (go - oa).norm().item() / oa.norm().item() <= 6e-2
+    assert ((gl - la).abs() / la.abs().clamp_min(1.0)).max().item() <= 1e-3
+    assert (go - ob).abs().max().item() <= 6e-2          # the stated fp8 bar, at the size it is stated for
