@@ -6,17 +6,19 @@
 // Work decomposition
 //   workgroup  = 256 Q rows of one (batch, q-head): 8 wavefronts x 32 rows, one workgroup per CU,
 //                two wavefronts per SIMD
-//   main loop  = 64-key tiles of the chunk, K and V double-buffered in LDS; wavefronts 0-3 stage K,
-//                wavefronts 4-7 stage V (transposed in registers with v_perm_b32 on the way)
+//   main loop  = 64-key tiles of the chunk.  K and V tiles go from global memory straight into LDS
+//                (buffer_load ... lds, no registers in between), row-major with the 16-byte chunks of
+//                a row XOR-swizzled, four stages each; every wavefront copies 8 rows of each tile
 //   S^T = K Q^T  : v_mfma_f32_32x32x16_bf16 with A = K rows (LDS), B = Q (registers, loaded once).
 //                  The accumulator layout puts one Q row in each lane (lane % 32) and 32 of the
 //                  64 keys of the tile in that lane's registers, so the online softmax needs one
 //                  exchange with lane ^ 32 per tile and no other cross-lane traffic.
 //   O^T = V^T P^T: the same lane that produced P^T[key][q] feeds it back as the B operand; the
-//                  key order inside one MFMA k-step is whatever the accumulator registers hold,
-//                  and V^T is written to LDS in exactly that key order, so P never moves.
+//                  key order inside one MFMA k-step is whatever the accumulator registers hold, and
+//                  the V^T operand is gathered in exactly that order from the row-major V tile by
+//                  ds_read_b64_tr_b16 (four keys of one head-dim column per lane), so P never moves.
 //   ping-pong    : every tile is split into a matrix phase (S^T of the next tile + O^T of this one,
-//                  32 MFMAs) and a vector phase (softmax of the next tile, LDS stores).  Wavefronts
+//                  32 MFMAs) and a vector phase (softmax of the next tile, tile copies).  Wavefronts
 //                  0-3 and 4-7 run half a tile apart, separated by workgroup barriers, so on every
 //                  SIMD one wavefront feeds the matrix pipe while the other does exponentials.
 #include "mhip_common.hpp"
@@ -28,13 +30,9 @@ constexpr int kD = 128;            // head dimension
 constexpr int kWaves = 8;
 constexpr int kBM = kWaves * 32;   // Q rows per workgroup
 constexpr int kBN = 64;            // keys per main-loop tile
-constexpr int kKStride = kD + 8;   // bf16 elements per K row in LDS (272 B: 16 B skew per row)
-constexpr int kVStride = kBN + 8;  // bf16 elements per V^T row in LDS (144 B)
-constexpr int kKBytes = kBN * kKStride * 2;   // 17408
-constexpr int kVBytes = kD * kVStride * 2;    // 18432
-constexpr int kKStages = 3;         // K(t+1) .. K(t+3) live while tile t is processed
-constexpr int kVStages = 2;
-constexpr int kVBase = kKStages * kKBytes;
+constexpr int kTileBytes = kBN * kD * 2;   // 16384: one K or V tile in LDS, 64 rows of 256 bytes
+constexpr int kStages = 4;                 // K(t+1) .. K(t+4) and V(t) .. V(t+3) live while tile t is processed
+constexpr int kVBase = kStages * kTileBytes;
 constexpr int kOStride = kD + 8;   // epilogue staging of O, bf16 elements per row
 #ifndef MHIP_FWD_PINGPONG
 #define MHIP_FWD_PINGPONG 1
@@ -63,9 +61,27 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
 }
 
+// The same descriptor as four scalar words, for the copies below.
+__device__ __forceinline__ u32x4 rsrc_words(const void* base, uint32_t bytes) {
+  const uint64_t a = (uint64_t)base;
+  u32x4 r;
+  r[0] = (uint32_t)a; r[1] = (uint32_t)(a >> 32) & 0xffffu; r[2] = bytes; r[3] = 0x00020000u;
+  return r;
+}
+
+// Global -> LDS copy of 16 bytes per lane without passing through registers: lane l's bytes land at LDS
+// address `lds_addr` + 16 l (wavefront-uniform base, in M0); lanes whose offset is out of the descriptor's
+// range write zeros.  Completion is counted by vmcnt.  Written as inline assembly so that the compiler's
+// own wait-count insertion does not see it: it would otherwise wait for all copies in flight before the
+// transposing LDS reads.  The waits are placed by hand where the loop needs them.
+__device__ __forceinline__ void copy16_to_lds(u32x4 rsrc, uint32_t lds_addr, int voffset, int soffset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+}
+
 template <bool CAUSAL>
 __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdParams p) {
-  __shared__ __attribute__((aligned(16))) unsigned char smem[kKStages * kKBytes + kVStages * kVBytes];
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kStages * kTileBytes];
 
   // Workgroup i runs on XCD i % 8.  Give every XCD a contiguous range of the (batch, head, q-tile)
   // order so that the workgroups sharing one K/V head also share one L2.
@@ -123,65 +139,68 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     for (int ks = 0; ks < 8; ++ks) asm volatile("" : "+v"(qf[ks]));
   }
 
-  // ---- global -> register staging of one K or V tile ----------------------------------------------
-  // K (waves 0-3): thread loads rows (lt/16 + 16 i), 16-byte chunk lt%16, lt = tid % 256.
-  // V (waves 4-7): thread loads the four rows of key quad lt/16, chunk lt%16 (8 head-dim values each).
-  // Per-thread byte offsets are fixed; the tile advances through the scalar offset of the load.
-  const int ld_chunk = tid & 15;
-  const int ld_row = (tid & 255) >> 4;
-  const uint16_t* gbase = group_b ? p.v + b * p.v_sb + hk * p.v_sh : p.k + b * p.k_sb + hk * p.k_sh;
-  const int64_t g_ss = group_b ? p.v_ss : p.k_ss;
-  const __amdgpu_buffer_rsrc_t grs = make_rsrc(gbase, (uint32_t)(((int64_t)(p.Sc - 1) * g_ss + kD) * 2));
-  int goff[4];
+  // ---- global -> LDS copies of the K and V tiles ---------------------------------------------------
+  // A tile is 64 rows of 256 bytes.  Chunk c (16 bytes) of row r lives at chunk position c ^ swz(r):
+  // the 32 rows a b128 operand read touches then spread over all banks, and so do the 8 rows x 4 chunks
+  // of a transposing read.  Wavefront w copies rows 8w .. 8w+7 of every tile with two instructions of
+  // 1 KB; lane l of instruction u lands at row 8w + 4u + l/16, position l%16 (the hardware places the
+  // lanes back to back) and therefore fetches chunk (l%16) ^ swz(row).  Rows past the end of the chunk
+  // are out of the descriptor's range and arrive as zeros.
+  auto swz = [](int row) { return ((row & 3) << 2) | ((row >> 2) & 3); };
+  const u32x4 krs = rsrc_words(p.k + b * p.k_sb + hk * p.k_sh, (uint32_t)(((int64_t)(p.Sc - 1) * p.k_ss + kD) * 2));
+  const u32x4 vrs = rsrc_words(p.v + b * p.v_sb + hk * p.v_sh, (uint32_t)(((int64_t)(p.Sc - 1) * p.v_ss + kD) * 2));
+  int kvoff[2], vvoff[2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
-    goff[i] = (int)((group_b ? ld_row * 4 + i : ld_row + 16 * i) * g_ss * 2) + ld_chunk * 16;
-  const int tile_bytes = (int)(kBN * g_ss * 2);
-  u32x4 greg[4];   // staging registers: a tile's loads are issued a whole tile before their LDS stores
-
-  auto load_tile = [&](int t) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) greg[i] = __builtin_amdgcn_raw_buffer_load_b128(grs, goff[i], t * tile_bytes, 0);
-  };
-
-  // LDS position of key quad (4 consecutive keys) inside a V^T row: MFMA k-step = quad / 4,
-  // lane half = quad % 2, first / second group of four accumulator registers = (quad % 4) / 2.
-  const int vt_off = ((ld_row >> 2) * 2 + (ld_row & 1)) * 16 + ((ld_row & 3) >> 1) * 8;
-  // Row d of V^T lives in LDS row d ^ rev3(d >> 4): the 16 lanes of one write (rows 8c + e, c = 0..15)
-  // and the 32 lanes of one read (rows 32 db + 0..31) then both spread over all banks.
-  const int vt_xor = ((ld_chunk >> 3) & 1) | (((ld_chunk >> 2) & 1) << 1) | (((ld_chunk >> 1) & 1) << 2);
-
-  auto store_tile = [&](int stage) {
-    if (!group_b) {
-      unsigned char* ks = smem + stage * kKBytes;
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        *reinterpret_cast<u32x4*>(ks + (ld_row + 16 * i) * (kKStride * 2) + ld_chunk * 16) = greg[i];
-    } else {
-      unsigned char* vs = smem + kVBase + stage * kVBytes;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        // dword j of each row holds head-dim values 2j (low half) and 2j+1 (high half)
-        u32x2 even, odd;
-        even[0] = __builtin_amdgcn_perm(greg[1][j], greg[0][j], 0x05040100u);
-        even[1] = __builtin_amdgcn_perm(greg[3][j], greg[2][j], 0x05040100u);
-        odd[0] = __builtin_amdgcn_perm(greg[1][j], greg[0][j], 0x07060302u);
-        odd[1] = __builtin_amdgcn_perm(greg[3][j], greg[2][j], 0x07060302u);
-        const int r0 = ld_chunk * 8 + ((2 * j) ^ vt_xor);
-        const int r1 = ld_chunk * 8 + ((2 * j + 1) ^ vt_xor);
-        *reinterpret_cast<u32x2*>(vs + r0 * (kVStride * 2) + vt_off) = even;
-        *reinterpret_cast<u32x2*>(vs + r1 * (kVStride * 2) + vt_off) = odd;
-      }
-    }
-  };
-
-  const int k_rd = ln * (kKStride * 2) + hf * 16;   // + mb*32*272 + ks*32
-  int v_rd[4];                                        // + kstep*32
-#pragma unroll
-  for (int db = 0; db < 4; ++db) {
-    const int x = (db >> 1) | ((db & 1) << 1) | ((ln >> 4) << 2);
-    v_rd[db] = (db * 32 + (ln ^ x)) * (kVStride * 2) + hf * 16;
+  for (int u = 0; u < 2; ++u) {
+    const int row = 8 * wave + 4 * u + (lane >> 4);
+    const int chunk = (lane & 15) ^ swz(row);
+    kvoff[u] = (int)(row * p.k_ss * 2) + chunk * 16;
+    vvoff[u] = (int)(row * p.v_ss * 2) + chunk * 16;
   }
+  const int k_tile_bytes = (int)(kBN * p.k_ss * 2);
+  const int v_tile_bytes = (int)(kBN * p.v_ss * 2);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem + wave * 2048;
+  auto copy_k = [&](int t, int stage) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) copy16_to_lds(krs, lds_base + stage * kTileBytes + u * 1024, kvoff[u], t * k_tile_bytes);
+  };
+  auto copy_v = [&](int t, int stage) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+      copy16_to_lds(vrs, lds_base + kVBase + stage * kTileBytes + u * 1024, vvoff[u], t * v_tile_bytes);
+  };
+
+  // K operand of S^T (A, 32 keys x 16 head-dim values): lane (ln, hf) reads chunk 2 kk + hf of row
+  // 32 mb + ln.
+  int k_rd[8];                                        // + mb * 8192
+#pragma unroll
+  for (int kk = 0; kk < 8; ++kk) k_rd[kk] = ln * 256 + (((2 * kk + hf) ^ swz(ln)) << 4);
+  // V^T operand of O^T (A, 32 head-dim values x 16 keys) for head-dim block db and k-step (mb, j2): the
+  // lane's 8 keys are rows R + {0..3} and R + 8 + {0..3}, R = 32 mb + 16 j2 + 4 hf -- the keys its P
+  // registers hold.  One ds_read_b64_tr_b16 per group of 4 rows: within 16 lanes, lane s supplies the
+  // address of row R + s/4, head-dim values 4 (s%4) .. +3 of the 16-column strip, and receives column s.
+  int v_rd[4][2];                                     // [db][second four rows]  + mb * 8192 + j2 * 4096
+  {
+    const int s16 = lane & 15, strip = (lane >> 4) & 1;
+    const int cl = 2 * strip + ((s16 & 3) >> 1);
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int row = 8 * h + 4 * hf + (s16 >> 2);
+        v_rd[db][h] = row * 256 + (((4 * db + cl) ^ swz(row)) << 4) + (s16 & 1) * 8;
+      }
+  }
+  typedef __attribute__((address_space(3))) bf16x4* lds_bf16x4;
+  auto read_k = [&](const unsigned char* ks, int mb, int kk) -> bf16x8 {
+    return *reinterpret_cast<const bf16x8*>(ks + k_rd[kk] + mb * 8192);
+  };
+  auto read_v = [&](const unsigned char* vs, int db, int kstep) -> bf16x8 {
+    const unsigned char* base = vs + (kstep >> 1) * 8192 + (kstep & 1) * 4096;
+    const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4)(base + v_rd[db][0]));
+    const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4)(base + v_rd[db][1]));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
   const int causal_shift = p.Sc - p.Sq;
 
   // ---- accumulators -----------------------------------------------------------------------------
@@ -201,7 +220,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
   bf16x8 pf[4];              // P^T of the current tile as bf16 B operands
 
   auto qk = [&](int stage) {
-    const unsigned char* ks = smem + stage * kKBytes;
+    const unsigned char* ks = smem + stage * kTileBytes;
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
@@ -210,19 +229,19 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     for (int kk = 0; kk < 8; ++kk) {
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb) {
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(ks + k_rd + mb * (32 * kKStride * 2) + kk * 32);
+        const bf16x8 kf = read_k(ks, mb, kk);
         s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], s[mb], 0, 0, 0);
       }
     }
   };
 
   auto pv = [&](int stage) {
-    const unsigned char* vs = smem + kVBase + stage * kVBytes;
+    const unsigned char* vs = smem + kVBase + stage * kTileBytes;
 #pragma unroll
     for (int kstep = 0; kstep < 4; ++kstep) {
 #pragma unroll
       for (int db = 0; db < 4; ++db) {
-        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vs + v_rd[db] + kstep * 32);
+        const bf16x8 vf = read_v(vs, db, kstep);
         o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kstep], o_acc[db], 0, 0, 0);
       }
     }
@@ -316,22 +335,21 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
   // Matrix phase of tile t: S^T(t+1) from K stage `ks_stage` and O^T += V^T(t) P^T(t) from V stage
   // `vs_stage`, 32 MFMAs fed by 32 LDS reads.  The reads run kFragDepth operands ahead of the MFMAs
   // through a ring of registers, so the LDS latency is covered by the MFMAs in between.
-  auto frag_addr = [&](int i, const unsigned char* ks, const unsigned char* vs) -> const bf16x8* {
-    if (i < 16) return reinterpret_cast<const bf16x8*>(ks + k_rd + (i & 1) * (32 * kKStride * 2) + (i >> 1) * 32);
-    const int j = i - 16;
-    return reinterpret_cast<const bf16x8*>(vs + v_rd[j & 3] + (j >> 2) * 32);
+  auto read_frag = [&](int i, const unsigned char* ks, const unsigned char* vs) -> bf16x8 {
+    if (i < 16) return read_k(ks, i & 1, i >> 1);
+    return read_v(vs, (i - 16) & 3, (i - 16) >> 2);
   };
   // The first kFragDepth operands (all of K) are read before the barrier that opens the phase, by
   // first_frags, so the matrix pipe starts without waiting for LDS.
   bf16x8 frag[kFragDepth];
   auto first_frags = [&](int ks_stage) {
-    const unsigned char* ks = smem + ks_stage * kKBytes;
+    const unsigned char* ks = smem + ks_stage * kTileBytes;
 #pragma unroll
-    for (int i = 0; i < kFragDepth; ++i) frag[i] = *frag_addr(i, ks, ks);
+    for (int i = 0; i < kFragDepth; ++i) frag[i] = read_frag(i, ks, ks);
   };
   auto matrix_phase = [&](int t_next, int ks_stage, int vs_stage) {
-    const unsigned char* ks = smem + ks_stage * kKBytes;
-    const unsigned char* vs = smem + kVBase + vs_stage * kVBytes;
+    const unsigned char* ks = smem + ks_stage * kTileBytes;
+    const unsigned char* vs = smem + kVBase + vs_stage * kTileBytes;
     const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
@@ -342,7 +360,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
         const int db = (i - 16) & 3, kstep = (i - 16) >> 2;
         o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag[i % kFragDepth], pf[kstep], o_acc[db], 0, 0, 0);
       }
-      if (i + kFragDepth < 32) frag[i % kFragDepth] = *frag_addr(i + kFragDepth, ks, vs);
+      if (i + kFragDepth < 32) frag[i % kFragDepth] = read_frag(i + kFragDepth, ks, vs);
       // S^T(t_next) is complete after slot 15; its softmax starts here, in the shadow of the O^T MFMAs
       if (i == 16) sm_mask(t_next);
       if (i >= 17 && i < 21) sm_max(i - 17);
@@ -353,45 +371,43 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
   };
 
   // ---- prologue: the first tiles into LDS, softmax of tile 0 -------------------------------------------
-  // K is staged three tiles ahead and V two: K(t+2) must be readable one phase before the matrix phase
-  // that consumes it, for first_frags.
-  const int lead = group_b ? kVStages : kKStages;
+  // Barriers inside the loop are bare s_barrier instructions: a fence would wait for every copy in flight.
   if (ntiles > 0) {
-    load_tile(0);
-    store_tile(0);
-    if (ntiles > 1) { load_tile(1); store_tile(1); }
-    if (!group_b && ntiles > 2) { load_tile(2); store_tile(2); }
-    if (lead < ntiles) load_tile(lead);   // lands during the first tile, stored in its vector phase
+#pragma unroll
+    for (int i = 0; i < kStages; ++i) copy_k(i, i);          // tiles past the chunk arrive as zeros
+#pragma unroll
+    for (int i = 0; i < kStages - 1; ++i) copy_v(i, i);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     qk(0);
     softmax_all(0);
     if (ntiles > 1) first_frags(1);
   }
   // Phase p of the main loop: group A (waves 0-3) runs the matrix phase of tile p/2 on even p and its
-  // vector phase on odd p; group B does the same one phase later.  K(t) lives in K stage t % 3, V(t) in V
-  // stage t & 1.  The vector phase of tile t stores K(t+3) over K(t) and V(t+2) over V(t): every wave has
-  // read K(t) in the matrix phase of tile t-1 and V(t) in the matrix phase of tile t.
-  if (kPingPong && group_b) __syncthreads();
-  int k3 = 0;   // t % 3
+  // vector phase on odd p; group B does the same one phase later.  K(t) and V(t) live in stage t % 4 of
+  // their rings.  In the vector phase of tile t every wavefront starts its share of the copies of K(t+4)
+  // (over K(t), last read in the matrix phase of tile t-1) and V(t+3) (over V(t-1)), and before the
+  // barrier that ends the phase waits for the copies it started one tile earlier: those are then visible
+  // to every wavefront two barriers later, in time for first_frags of K(t+3) and the matrix phase of V(t+2).
+  if (kPingPong && group_b) __builtin_amdgcn_s_barrier();
   for (int t = 0; t + 1 < ntiles; ++t) {
-    const int k3n = k3 == 2 ? 0 : k3 + 1;          // (t+1) % 3
     // ---- matrix phase: S^T(t+1) = K(t+1) Q^T and O^T += V^T(t) P^T(t), first part of softmax(t+1) ------
     __builtin_amdgcn_s_setprio(2);
-    matrix_phase(t + 1, k3n, t & 1);
+    matrix_phase(t + 1, (t + 1) & 3, t & 3);
     __builtin_amdgcn_s_setprio(0);
-    __syncthreads();
-    // ---- vector phase: rest of softmax(t+1), this wave's share of the next tiles into LDS ------------------
+    __builtin_amdgcn_s_barrier();
+    // ---- vector phase: rest of softmax(t+1), copies of the tiles ahead -------------------------------------
 #pragma unroll
     for (int e = kEarly; e < 16; ++e) sm_exp(e);
     sm_finish();
-    if (t + lead < ntiles) store_tile(group_b ? (t & 1) : k3);   // loaded a tile ago
-    if (t + lead + 1 < ntiles) load_tile(t + lead + 1);           // a whole tile to land
-    if (t + 2 < ntiles) first_frags(k3n == 2 ? 0 : k3n + 1);      // K(t+2), for the next matrix phase
-    k3 = k3n;
-    __syncthreads();
+    copy_k(t + 4, t & 3);
+    copy_v(t + 3, (t + 3) & 3);
+    if (t + 2 < ntiles) first_frags((t + 2) & 3);             // K(t+2), for the next matrix phase
+    asm volatile("s_waitcnt vmcnt(4)" ::: "memory");          // the four copies of one tile ago are done
+    __builtin_amdgcn_s_barrier();
   }
-  if (ntiles > 0) pv((ntiles - 1) & 1);             // last tile: nothing left to prefetch or exponentiate
-  if (kPingPong && !group_b) __syncthreads();
+  if (ntiles > 0) pv((ntiles - 1) & 3);             // last tile: nothing left to prefetch or exponentiate
+  if (kPingPong && !group_b) __builtin_amdgcn_s_barrier();
 
   // ---- epilogue -----------------------------------------------------------------------------------
   const float l_tot = pair_sum(l_run);
@@ -401,6 +417,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     p.lse[((int64_t)b * p.Hq + hq) * p.Sq + my_q] = lse;
   }
 
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // zero-filled copies of tiles past the end included
   __syncthreads();   // every wave is done with the K/V tiles: reuse LDS to transpose O
   unsigned char* os = smem + wave * (32 * kOStride * 2);
 #pragma unroll
