@@ -5,7 +5,8 @@
 //     dV = P^T dout,  dP = dout v^T,  dS = P * (dP - delta),  dQ = scale * dS k,  dK = scale * dS^T q
 //
 // Three kernels, no atomics (so every run is deterministic):
-//   bwd_delta    delta[b,h,i] = sum_d dout * out                        (bandwidth bound)
+//   bwd_prepare  delta[b,h,i] = sum_d dout * out and lse2 = lse * log2(e), with -inf (a row that saw no
+//                key) turned into +inf so that P = exp2(s - lse2) = 0 there       (bandwidth bound)
 //   bwd_main<DQ=false>  one workgroup per 128 keys of one KV head: K and V rows stay in registers,
 //                Q / dout tiles of the (grouped) query heads stream through LDS; accumulates dK, dV
 //   bwd_main<DQ=true>   one workgroup per 128 query rows of one head: Q and dout rows stay in registers,
@@ -15,8 +16,11 @@
 //     T1[c][r] = X_str[c] . X_st[r]      (scores)          T2[c][r] = Y_str[c] . Y_st[r]      (dP)
 //     acc^T[d][r] += X_str^T[d][c] dS[c][r]                (dQ or dK)
 //     acc2^T[d][r] += Y_str^T[d][c] P[c][r]                (dV, DQ=false only)
-// so P and dS feed the second MFMA straight from the accumulator registers, and the transposed
-// streamed tiles are written to LDS in the matching key order (v_perm_b32 transposition in registers).
+// so P and dS feed the second MFMA straight from the accumulator registers.  The streamed tiles are
+// copied global -> LDS without registers in between (buffer_load ... lds), row-major with swizzled
+// 16-byte chunks, four stages deep; T1 / T2 read them with ds_read_b128 and the transposed operands
+// of the second MFMAs are gathered from the same tiles with ds_read_b64_tr_b16, in the key order the
+// accumulator registers hold.
 #include "mhip_common.hpp"
 
 namespace mhip {
@@ -25,18 +29,17 @@ namespace {
 constexpr int kD = 128;
 constexpr int kTile = 64;             // streamed rows per main-loop tile
 constexpr int kRowsPerWg = 128;       // stationary rows per workgroup (4 wavefronts x 32)
-constexpr int kRmStride = kD + 8;     // row-major tile: bf16 per row (272 B)
-constexpr int kTrStride = kTile + 8;  // transposed tile: bf16 per row (144 B)
-constexpr int kRmBytes = kTile * kRmStride * 2;   // 17408
-constexpr int kTrBytes = kD * kTrStride * 2;      // 18432
-constexpr int kOffX = 0, kOffY = kRmBytes, kOffXT = 2 * kRmBytes, kOffYT = 2 * kRmBytes + kTrBytes;
-constexpr int kOffLse = 2 * kRmBytes + 2 * kTrBytes, kOffDelta = kOffLse + kTile * 4;
-constexpr int kSmemBytes = kOffDelta + kTile * 4;  // 72192
+constexpr int kTileBytes = kTile * kD * 2;             // 16384: 64 rows of 256 bytes
+constexpr int kOffY = kTileBytes, kOffLse = 2 * kTileBytes, kOffDelta = kOffLse + kTile * 4;
+constexpr int kStageBytes = kOffDelta + kTile * 4;     // X tile, Y tile, lse2 and delta of the streamed rows
+constexpr int kStages = 4;
+constexpr int kSmemBytes = kStages * kStageBytes;      // 133120
 constexpr int kOStride = kD + 8;
+constexpr int kNoTile = 0x7fff0000;   // scalar offset that puts every lane of a copy out of range
 
 struct BwdParams {
   const uint16_t* q; const uint16_t* k; const uint16_t* v; const uint16_t* dout;
-  const float* lse; const float* delta;
+  const float* lse2; const float* delta;   // both (B, Hq, Sq) fp32, written by bwd_prepare
   uint16_t* dq; uint16_t* dk; uint16_t* dv; float* dq_acc;
   int B, Sq, Sc, Hq, Hkv, group;
   int64_t q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, dk_sb, dk_ss, dk_sh;
@@ -47,24 +50,20 @@ struct BwdParams {
   int heads_per_xcd;   // (batch, stationary head) pairs per XCD when they divide evenly, else 0
 };
 
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
-}
-
-// delta = rowsum(dout * out): one row of 128 values per 16 lanes (8 values each)
-__global__ __launch_bounds__(256) void bwd_delta(const uint16_t* __restrict__ dout, const uint16_t* __restrict__ out,
-                                                 float* __restrict__ delta, int B, int Sq, int Hq,
-                                                 int64_t sb, int64_t ss, int64_t sh) {
+// delta = rowsum(dout * out): one row of 128 values per 16 lanes (8 values each); lse2 as described above
+__global__ __launch_bounds__(256) void bwd_prepare(const uint16_t* __restrict__ dout, const uint16_t* __restrict__ out,
+                                                   const float* __restrict__ lse, float* __restrict__ delta,
+                                                   float* __restrict__ lse2, int B, int Sq, int Hq,
+                                                   int64_t sb, int64_t ss, int64_t sh) {
   const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   const int64_t rows = (int64_t)B * Hq * Sq;
   const int c = threadIdx.x & 15;
   float acc = 0.f;
-  int b = 0, h = 0, s = 0;
   if (row < rows) {
-    s = (int)(row % Sq);
+    const int s = (int)(row % Sq);
     const int64_t bh = row / Sq;
-    h = (int)(bh % Hq);
-    b = (int)(bh / Hq);
+    const int h = (int)(bh % Hq);
+    const int b = (int)(bh / Hq);
     const int64_t off = b * sb + (int64_t)s * ss + h * sh + c * 8;
     const u32x4 a = *reinterpret_cast<const u32x4*>(dout + off);
     const u32x4 o = *reinterpret_cast<const u32x4*>(out + off);
@@ -73,7 +72,11 @@ __global__ __launch_bounds__(256) void bwd_delta(const uint16_t* __restrict__ do
   }
 #pragma unroll
   for (int m = 8; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 16);
-  if (row < rows && c == 0) delta[row] = acc;      // (B, Hq, Sq) contiguous
+  if (row < rows && c == 0) {      // (B, Hq, Sq) contiguous
+    delta[row] = acc;
+    const float l = lse[row];
+    lse2[row] = (l == -INFINITY) ? INFINITY : l * kLog2e;
+  }
 }
 
 template <bool DQ, bool CAUSAL>
@@ -137,14 +140,15 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) { asm volatile("" : "+v"(xf[ks])); asm volatile("" : "+v"(yf[ks])); }
   }
-  // DQ: the query is the stationary row, its lse / delta are per-lane scalars
+  // DQ: the query is the stationary row, its lse2 / delta are per-lane scalars
   float lse2_lane = 0.f, delta_lane = 0.f;
   if (DQ) {
     const int row = my_r < n_st ? my_r : n_st - 1;
-    const float l = p.lse[((int64_t)b * p.Hq + hs) * p.Sq + row];
-    lse2_lane = (l == -INFINITY) ? INFINITY : l * kLog2e;     // rows that saw no key: P = 0
+    lse2_lane = p.lse2[((int64_t)b * p.Hq + hs) * p.Sq + row];
     delta_lane = p.delta[((int64_t)b * p.Hq + hs) * p.Sq + row];
   }
+  // pin the prologue loads here: the copies below are invisible to the compiler's wait counting
+  asm volatile("" : "+v"(lse2_lane), "+v"(delta_lane));
 
   // ---- streamed tiles ---------------------------------------------------------------------------------
   // DQ: K / V rows of kv head hs / group.  Otherwise: Q / dout rows of the `group` query heads that share
@@ -165,8 +169,6 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
   const int span = tiles_per_head - first_tile;
   const int ntiles = span * heads_str;
 
-  const int ld_chunk = tid & 15;
-  const int ld_quad = tid >> 4;                       // rows 4 quad .. 4 quad + 3 of the tile
   const uint16_t* xbase; const uint16_t* ybase; int64_t s_ss, s_sh; uint32_t s_bytes;
   if (DQ) {
     const int hk = hs / p.group;
@@ -178,83 +180,71 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     s_ss = p.q_ss; s_sh = p.q_sh;
     s_bytes = (uint32_t)(((int64_t)(p.Sq - 1) * p.q_ss + (int64_t)(p.Hq - 1) * p.q_sh + kD) * 2);
   }
-  const __amdgpu_buffer_rsrc_t xrs = make_rsrc(xbase, s_bytes);
-  const __amdgpu_buffer_rsrc_t yrs = make_rsrc(ybase, s_bytes);
-  int goff[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) goff[i] = (int)((ld_quad * 4 + i) * s_ss * 2) + ld_chunk * 16;
-  u32x4 xreg[4], yreg[4];
-  float lse_reg = 0.f, delta_reg = 0.f;
+  const u32x4 xrs = rsrc_words(xbase, s_bytes);
+  const u32x4 yrs = rsrc_words(ybase, s_bytes);
 
   // tile index -> (head of the group, first streamed row)
   auto tile_head = [&](int t) { return DQ ? 0 : t / span; };
   auto tile_row0 = [&](int t) { return (first_tile + (DQ ? t : t % span)) * kTile; };
 
-  auto load_tile = [&](int t) {
-    const int hq = DQ ? 0 : hs * p.group + tile_head(t);
-    const int c0 = tile_row0(t);
-    const int soff = (int)(((int64_t)c0 * s_ss + (int64_t)hq * s_sh) * 2);
+  // Wavefront w copies rows 16w .. 16w+15 of the X and the Y tile: four instructions of 1 KB each; lane l
+  // of instruction u lands at row 16w + 4u + l/16, chunk position l%16, and fetches the chunk that lives
+  // there.  Rows past the end of the streamed tensor arrive as zeros when the layout puts them past the
+  // descriptor's range, and their P / dS are zeroed by index in any case.  lse2 and delta of the 64
+  // streamed rows (DQ=false) are copied by the even / odd wavefronts (twice the same bytes: every
+  // wavefront then has the same number of copies in flight, which the vmcnt waits rely on).
+  int cvoff[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      xreg[i] = __builtin_amdgcn_raw_buffer_load_b128(xrs, goff[i], soff, 0);
-      yreg[i] = __builtin_amdgcn_raw_buffer_load_b128(yrs, goff[i], soff, 0);
-    }
-    if (!DQ && tid < kTile) {
-      const int i = c0 + tid;
-      if (i < p.Sq) {
-        const float l = p.lse[((int64_t)b * p.Hq + hq) * p.Sq + i];
-        lse_reg = (l == -INFINITY) ? INFINITY : l * kLog2e;
-        delta_reg = p.delta[((int64_t)b * p.Hq + hq) * p.Sq + i];
-      } else {
-        lse_reg = INFINITY;     // rows past the end of the shard: P = 0
-        delta_reg = 0.f;
-      }
-    }
-  };
-
-  // transposed tiles use the layout of V^T in the forward kernel: row d of the tile lives in LDS row
-  // d ^ rev3(d >> 4), and inside a row the streamed rows are ordered the way the accumulator registers
-  // of one MFMA k-step hold them
-  const int tr_off = ((ld_quad >> 2) * 2 + (ld_quad & 1)) * 16 + ((ld_quad & 3) >> 1) * 8;
-  const int tr_xor = ((ld_chunk >> 3) & 1) | (((ld_chunk >> 2) & 1) << 1) | (((ld_chunk >> 1) & 1) << 2);
-  auto store_transposed = [&](unsigned char* dst, const u32x4 (&reg)[4]) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      u32x2 even, odd;
-      even[0] = __builtin_amdgcn_perm(reg[1][j], reg[0][j], 0x05040100u);
-      even[1] = __builtin_amdgcn_perm(reg[3][j], reg[2][j], 0x05040100u);
-      odd[0] = __builtin_amdgcn_perm(reg[1][j], reg[0][j], 0x07060302u);
-      odd[1] = __builtin_amdgcn_perm(reg[3][j], reg[2][j], 0x07060302u);
-      const int r_even = ld_chunk * 8 + ((2 * j) ^ tr_xor);
-      const int r_odd = ld_chunk * 8 + ((2 * j + 1) ^ tr_xor);
-      *reinterpret_cast<u32x2*>(dst + r_even * (kTrStride * 2) + tr_off) = even;
-      *reinterpret_cast<u32x2*>(dst + r_odd * (kTrStride * 2) + tr_off) = odd;
-    }
-  };
-  auto store_tile = [&]() {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int off = (ld_quad * 4 + i) * (kRmStride * 2) + ld_chunk * 16;
-      *reinterpret_cast<u32x4*>(smem + kOffX + off) = xreg[i];
-      *reinterpret_cast<u32x4*>(smem + kOffY + off) = yreg[i];
-    }
-    store_transposed(smem + kOffXT, xreg);
-    if (!DQ) {
-      store_transposed(smem + kOffYT, yreg);
-      if (tid < kTile) {
-        reinterpret_cast<float*>(smem + kOffLse)[tid] = lse_reg;
-        reinterpret_cast<float*>(smem + kOffDelta)[tid] = delta_reg;
-      }
-    }
-  };
-
-  const int rm_rd = ln * (kRmStride * 2) + hf * 16;      // + mb*32*272 + kk*32
-  int tr_rd[4];                                            // + kstep*32
-#pragma unroll
-  for (int db = 0; db < 4; ++db) {
-    const int x = (db >> 1) | ((db & 1) << 1) | ((ln >> 4) << 2);
-    tr_rd[db] = (db * 32 + (ln ^ x)) * (kTrStride * 2) + hf * 16;
+  for (int u = 0; u < 4; ++u) {
+    const int row = 16 * wave + 4 * u + (lane >> 4);
+    cvoff[u] = (int)(row * s_ss * 2) + (((lane & 15) ^ lds_row_swizzle(row)) << 4);
   }
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
+  auto copy_tile = [&](int t, int stage) {
+    const bool live = t < ntiles;
+    const int hq = DQ ? 0 : hs * p.group + tile_head(live ? t : 0);
+    const int c0 = tile_row0(live ? t : 0);
+    const int soff = live ? (int)(((int64_t)c0 * s_ss + (int64_t)hq * s_sh) * 2) : kNoTile;
+    const uint32_t dst = lds_base + stage * kStageBytes + wave * 4096;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) copy16_to_lds(xrs, dst + u * 1024, cvoff[u], soff);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) copy16_to_lds(yrs, dst + kOffY + u * 1024, cvoff[u], soff);
+    if (!DQ) {
+      const float* src = ((wave & 1) ? p.delta : p.lse2) + ((int64_t)b * p.Hq + hq) * p.Sq;
+      copy4_to_lds(rsrc_words(src, (uint32_t)p.Sq * 4u), lds_base + stage * kStageBytes + ((wave & 1) ? kOffDelta : kOffLse),
+                   lane * 4, live ? c0 * 4 : kNoTile);
+    }
+  };
+  constexpr int kCopiesPerTile = DQ ? 8 : 9;
+
+  // row-major operand reads (A of T1 / T2): lane (ln, hf) reads chunk 2 kk + hf of row 32 mb + ln
+  int rm_rd[8];                                       // + mb * 8192
+#pragma unroll
+  for (int kk = 0; kk < 8; ++kk) rm_rd[kk] = ln * 256 + (((2 * kk + hf) ^ lds_row_swizzle(ln)) << 4);
+  // transposed operand reads (A of the second MFMAs) for head-dim block db and k-step (mb, j2): the lane's
+  // 8 streamed rows are R + {0..3} and R + 8 + {0..3}, R = 32 mb + 16 j2 + 4 hf -- the rows its P / dS
+  // registers hold.  One ds_read_b64_tr_b16 per group of 4 rows: within 16 lanes, lane s supplies the
+  // address of row R + s/4, head-dim values 4 (s%4) .. +3 of the 16-column strip, and receives column s.
+  int tr_rd[4][2];                                    // [db][second four rows]  + mb * 8192 + j2 * 4096
+  {
+    const int s16 = lane & 15, strip = (lane >> 4) & 1;
+    const int cl = 2 * strip + ((s16 & 3) >> 1);
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int row = 8 * h + 4 * hf + (s16 >> 2);
+        tr_rd[db][h] = row * 256 + (((4 * db + cl) ^ lds_row_swizzle(row)) << 4) + (s16 & 1) * 8;
+      }
+  }
+  typedef __attribute__((address_space(3))) bf16x4* lds_bf16x4;
+  auto read_tr = [&](const unsigned char* tile, int db, int kstep) -> bf16x8 {
+    const unsigned char* base = tile + (kstep >> 1) * 8192 + (kstep & 1) * 4096;
+    const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4)(base + tr_rd[db][0]));
+    const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4)(base + tr_rd[db][1]));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
 
   f32x16 acc1[4], acc2[4];      // DQ: acc1 = dQ^T.  Otherwise acc1 = dK^T, acc2 = dV^T
 #pragma unroll
@@ -263,85 +253,138 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     for (int j = 0; j < 16; ++j) { acc1[i][j] = 0.f; acc2[i][j] = 0.f; }
   const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-  if (ntiles > 0) load_tile(0);
-  for (int t = 0; t < ntiles; ++t) {
-    __syncthreads();                 // everybody is done reading the previous tile
-    store_tile();
-    if (t + 1 < ntiles) load_tile(t + 1);
-    __syncthreads();
-
-    // ---- T1 = X_str X_st^T (scores), T2 = Y_str Y_st^T (dP): 64 streamed x 32 stationary rows ----------
-    f32x16 t1[2], t2[2];
+  // Tile t lives in stage t % 4.  One step works on two tiles: the 32 MFMAs of T1 / T2 of tile t+1 are
+  // issued interleaved with the exponentials of tile t (whose T1 / T2 the step before left in registers),
+  // then the MFMAs that accumulate tile t follow.  A step starts by waiting for this wavefront's copies
+  // of tile t+1 (those of tile t+2 stay in flight) and a barrier: after it tile t+1 is complete for every
+  // wavefront and nobody reads tile t-1 any more, whose stage then receives tile t+3.  Tiles past the end
+  // are copied as zeros (and their T1 / T2 computed, unused) so that the number of copies in flight
+  // stays the same.
+  constexpr int kDepth = 4;                                // operand reads in flight ahead of the MFMAs
+  auto read_rm = [&](const unsigned char* xs, int i) -> bf16x8 {        // slot i of the T1 / T2 sequence
+    const int kk = i >> 2, mb = (i >> 1) & 1;
+    return *reinterpret_cast<const bf16x8*>(xs + ((i & 1) ? kOffY : 0) + rm_rd[kk] + mb * 8192);
+  };
+  auto t_mfma = [&](int i, const bf16x8& a, f32x16 (&n1)[2], f32x16 (&n2)[2]) {
+    const int kk = i >> 2, mb = (i >> 1) & 1;
+    if (i & 1) n2[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, yf[kk], kk == 0 ? zero : n2[mb], 0, 0, 0);
+    else n1[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, xf[kk], kk == 0 ? zero : n1[mb], 0, 0, 0);
+  };
+  // T1 / T2 of one tile without anything interleaved (first tile)
+  auto t_only = [&](int stage, f32x16 (&n1)[2], f32x16 (&n2)[2]) {
+    const unsigned char* xs = smem + stage * kStageBytes;
+    bf16x8 ring[kDepth];
 #pragma unroll
-    for (int kk = 0; kk < 8; ++kk) {
+    for (int i = 0; i < kDepth; ++i) ring[i] = read_rm(xs, i);
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb) {
-        const int off = rm_rd + mb * (32 * kRmStride * 2) + kk * 32;
-        const bf16x8 xa = *reinterpret_cast<const bf16x8*>(smem + kOffX + off);
-        const bf16x8 ya = *reinterpret_cast<const bf16x8*>(smem + kOffY + off);
-        t1[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa, xf[kk], kk == 0 ? zero : t1[mb], 0, 0, 0);
-        t2[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ya, yf[kk], kk == 0 ? zero : t2[mb], 0, 0, 0);
-      }
+    for (int i = 0; i < 32; ++i) {
+      t_mfma(i, ring[i % kDepth], n1, n2);
+      if (i + kDepth < 32) ring[i % kDepth] = read_rm(xs, i + kDepth);
     }
+  };
+  bf16x8 pfrag[4], dsfrag[4];
+  // P and dS of element j (accumulator register) of block mb of the current tile, in place
+  auto p_ds = [&](int mb, int j, const f32x4& lv, const f32x4& dv, f32x16 (&c1)[2], f32x16 (&c2)[2],
+                  bool need_mask, int c0) {
+    const int g = j >> 2, e = j & 3;
+    const float l = DQ ? lse2_lane : lv[e];
+    const float d = DQ ? delta_lane : dv[e];
+    float pe = fast_exp2(__builtin_fmaf(c1[mb][j], p.scale_log2, -l));
+    if (need_mask) {
+      const int c = c0 + mb * 32 + g * 8 + hf * 4 + e;     // streamed row of this element
+      bool hidden = c >= n_str;
+      if (CAUSAL) hidden = hidden || (DQ ? (c > my_r + shift) : (my_r > c + shift));
+      if (hidden) pe = 0.f;
+    }
+    c1[mb][j] = pe;
+    c2[mb][j] = pe * (c2[mb][j] - d);
+  };
+  auto pack_frags = [&](int mb, int j2, const f32x16 (&c1)[2], const f32x16 (&c2)[2]) {
+    u32x4 wp, wd;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      wp[e] = pack_bf16(c1[mb][8 * j2 + 2 * e], c1[mb][8 * j2 + 2 * e + 1]);
+      wd[e] = pack_bf16(c2[mb][8 * j2 + 2 * e], c2[mb][8 * j2 + 2 * e + 1]);
+    }
+    pfrag[mb * 2 + j2] = __builtin_bit_cast(bf16x8, wp);
+    dsfrag[mb * 2 + j2] = __builtin_bit_cast(bf16x8, wd);
+  };
 
-    // ---- P = exp2(scale_log2 T1 - lse log2e), dS = P (T2 - delta), hidden elements -> 0 ----------------
+  auto step = [&](int t, f32x16 (&c1)[2], f32x16 (&c2)[2], f32x16 (&n1)[2], f32x16 (&n2)[2]) {
+    if (DQ) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+    static_assert(kCopiesPerTile == (DQ ? 8 : 9), "the vmcnt immediates are one tile of copies");
+    __builtin_amdgcn_s_barrier();
+    copy_tile(t + 3, (t + 3) & 3);
+    const unsigned char* xs = smem + (t & 3) * kStageBytes;            // tile t
+    const unsigned char* xn = smem + ((t + 1) & 3) * kStageBytes;      // tile t+1
     const int c0 = tile_row0(t);
-    bf16x8 pfrag[4], dsfrag[4];
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb) {
-      float pv[16], dsv[16];
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        float l4[4], d4[4];
-        if (DQ) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) { l4[e] = lse2_lane; d4[e] = delta_lane; }
-        } else {
-          const int row = mb * 32 + g * 8 + hf * 4;
-          const f32x4 lv = *reinterpret_cast<const f32x4*>(smem + kOffLse + row * 4);
-          const f32x4 dv = *reinterpret_cast<const f32x4*>(smem + kOffDelta + row * 4);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) { l4[e] = lv[e]; d4[e] = dv[e]; }
-        }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int j = g * 4 + e;
-          const int c = c0 + mb * 32 + g * 8 + hf * 4 + e;       // streamed row of this element
-          float pe = fast_exp2(__builtin_fmaf(t1[mb][j], p.scale_log2, -l4[e]));
-          bool hidden = DQ ? (c >= p.Sc) : false;                 // keys past the chunk (zero filled)
-          if (CAUSAL) hidden = hidden || (DQ ? (c > my_r + shift) : (my_r > c + shift));
-          if (hidden) pe = 0.f;
-          pv[j] = pe;
-          dsv[j] = pe * (t2[mb][j] - d4[e]);
-        }
-      }
-#pragma unroll
-      for (int j2 = 0; j2 < 2; ++j2) {
-        u32x4 wp, wd;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          wp[e] = pack_bf16(pv[8 * j2 + 2 * e], pv[8 * j2 + 2 * e + 1]);
-          wd[e] = pack_bf16(dsv[8 * j2 + 2 * e], dsv[8 * j2 + 2 * e + 1]);
-        }
-        pfrag[mb * 2 + j2] = __builtin_bit_cast(bf16x8, wp);
-        dsfrag[mb * 2 + j2] = __builtin_bit_cast(bf16x8, wd);
-      }
-    }
+    bool need_mask = c0 + kTile > n_str;                       // rows past the end of the streamed tensor
+    if (CAUSAL) need_mask = need_mask || (DQ ? (c0 + kTile - 1 > r0 + shift) : (r0 + kRowsPerWg - 1 > c0 + shift));
 
-    // ---- acc1^T += X_str^T dS,  acc2^T += Y_str^T P ------------------------------------------------------
+    // ---- T1 / T2 of tile t+1 (slot i = one MFMA), P / dS of tile t (slot i = element i % 16 of block i / 16) ----
+    {
+      bf16x8 ring[kDepth];
 #pragma unroll
-    for (int kstep = 0; kstep < 4; ++kstep) {
+      for (int i = 0; i < kDepth; ++i) ring[i] = read_rm(xn, i);
+      f32x4 lv = {0.f, 0.f, 0.f, 0.f}, dv = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int db = 0; db < 4; ++db) {
-        const bf16x8 xt = *reinterpret_cast<const bf16x8*>(smem + kOffXT + tr_rd[db] + kstep * 32);
-        acc1[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xt, dsfrag[kstep], acc1[db], 0, 0, 0);
-        if (!DQ) {
-          const bf16x8 yt = *reinterpret_cast<const bf16x8*>(smem + kOffYT + tr_rd[db] + kstep * 32);
-          acc2[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(yt, pfrag[kstep], acc2[db], 0, 0, 0);
+      for (int i = 0; i < 32; ++i) {
+        t_mfma(i, ring[i % kDepth], n1, n2);
+        if (i + kDepth < 32) ring[i % kDepth] = read_rm(xn, i + kDepth);
+        const int mb = i >> 4, j = i & 15;
+        if (!DQ && (j & 3) == 0) {
+          const int row = mb * 32 + (j >> 2) * 8 + hf * 4;
+          lv = *reinterpret_cast<const f32x4*>(xs + kOffLse + row * 4);
+          dv = *reinterpret_cast<const f32x4*>(xs + kOffDelta + row * 4);
         }
+        p_ds(mb, j, lv, dv, c1, c2, need_mask, c0);
+        if ((j & 7) == 7) pack_frags(mb, j >> 3, c1, c2);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
+    // ---- acc1^T += X_str^T dS,  acc2^T += Y_str^T P  (tile t) ---------------------------------------------
+    {
+      constexpr int kN = DQ ? 16 : 32;
+      auto read_acc = [&](int i) -> bf16x8 {
+        const int m = DQ ? i : (i >> 1);
+        const int db = m & 3, kstep = m >> 2;
+        return read_tr((DQ || !(i & 1)) ? xs : xs + kOffY, db, kstep);
+      };
+      bf16x8 ring[kDepth];
+#pragma unroll
+      for (int i = 0; i < kDepth; ++i) ring[i] = read_acc(i);
+#pragma unroll
+      for (int i = 0; i < kN; ++i) {
+        const int m = DQ ? i : (i >> 1);
+        const int db = m & 3, kstep = m >> 2;
+        if (DQ || !(i & 1)) acc1[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % kDepth], dsfrag[kstep], acc1[db], 0, 0, 0);
+        else acc2[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % kDepth], pfrag[kstep], acc2[db], 0, 0, 0);
+        if (i + kDepth < kN) ring[i % kDepth] = read_acc(i + kDepth);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+
+  f32x16 ta1[2], ta2[2], tb1[2], tb2[2];
+  if (ntiles > 0) {
+    copy_tile(0, 0);
+    copy_tile(1, 1);
+    copy_tile(2, 2);
+    if (DQ) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    t_only(0, ta1, ta2);
   }
+  {
+    int t = 0;
+    for (; t + 1 < ntiles; t += 2) {
+      step(t, ta1, ta2, tb1, tb2);
+      step(t + 1, tb1, tb2, ta1, ta2);
+    }
+    if (t < ntiles) step(t, ta1, ta2, tb1, tb2);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the zero-filled copies of tiles past the end
 
   // ---- epilogue: acc^T[d][r] -> rows of the output through LDS --------------------------------------------
   auto write_out = [&](const f32x16 (&acc)[4], float mul, uint16_t* dst, int64_t d_sb, int64_t d_ss,
@@ -400,7 +443,7 @@ using namespace mhip;
 extern "C" int64_t mhip_attn_bwd_workspace_bytes(int B, int Sq, int Sc, int Hq, int Hkv, int D) {
   (void)Sc; (void)Hkv; (void)D;
   if (B < 0 || Sq < 0 || Hq < 0) return 0;
-  return (int64_t)B * Hq * Sq * 4 + 16;     // delta (B, Hq, Sq) fp32
+  return (int64_t)B * Hq * Sq * 8 + 32;     // delta and lse2, (B, Hq, Sq) fp32 each
 }
 
 extern "C" int mhip_attn_bwd_block(const void* dout, const void* q, const void* k, const void* v,
@@ -435,7 +478,9 @@ extern "C" int mhip_attn_bwd_block(const void* dout, const void* q, const void* 
   BwdParams p;
   p.q = static_cast<const uint16_t*>(q); p.k = static_cast<const uint16_t*>(k);
   p.v = static_cast<const uint16_t*>(v); p.dout = static_cast<const uint16_t*>(dout);
-  p.lse = lse; p.delta = static_cast<const float*>(workspace);
+  float* delta_buf = static_cast<float*>(workspace);
+  float* lse2_buf = delta_buf + (((int64_t)B * Hq * Sq + 3) & ~int64_t(3));     // 16-byte aligned
+  p.lse2 = lse2_buf; p.delta = delta_buf;
   p.dq = static_cast<uint16_t*>(dq); p.dk = static_cast<uint16_t*>(dk); p.dv = static_cast<uint16_t*>(dv);
   p.dq_acc = dq_acc;
   p.B = B; p.Sq = Sq; p.Sc = Sc; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv;
@@ -447,9 +492,9 @@ extern "C" int mhip_attn_bwd_block(const void* dout, const void* q, const void* 
 
   if (Sq > 0) {
     const int64_t rows = (int64_t)B * Hq * Sq;
-    hipLaunchKernelGGL(bwd_delta, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
-                       static_cast<const uint16_t*>(dout), static_cast<const uint16_t*>(out),
-                       static_cast<float*>(workspace), B, Sq, Hq, q_sb, q_ss, q_sh);
+    hipLaunchKernelGGL(bwd_prepare, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
+                       static_cast<const uint16_t*>(dout), static_cast<const uint16_t*>(out), lse,
+                       delta_buf, lse2_buf, B, Sq, Hq, q_sb, q_ss, q_sh);
     // dQ: one workgroup per 128 query rows
     p.n_tiles = (Sq + kRowsPerWg - 1) / kRowsPerWg;
     p.total = B * Hq * p.n_tiles;

@@ -61,24 +61,6 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
 }
 
-// The same descriptor as four scalar words, for the copies below.
-__device__ __forceinline__ u32x4 rsrc_words(const void* base, uint32_t bytes) {
-  const uint64_t a = (uint64_t)base;
-  u32x4 r;
-  r[0] = (uint32_t)a; r[1] = (uint32_t)(a >> 32) & 0xffffu; r[2] = bytes; r[3] = 0x00020000u;
-  return r;
-}
-
-// Global -> LDS copy of 16 bytes per lane without passing through registers: lane l's bytes land at LDS
-// address `lds_addr` + 16 l (wavefront-uniform base, in M0); lanes whose offset is out of the descriptor's
-// range write zeros.  Completion is counted by vmcnt.  Written as inline assembly so that the compiler's
-// own wait-count insertion does not see it: it would otherwise wait for all copies in flight before the
-// transposing LDS reads.  The waits are placed by hand where the loop needs them.
-__device__ __forceinline__ void copy16_to_lds(u32x4 rsrc, uint32_t lds_addr, int voffset, int soffset) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-               :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
-}
-
 template <bool CAUSAL>
 __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdParams p) {
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kStages * kTileBytes];
@@ -146,7 +128,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
   // 1 KB; lane l of instruction u lands at row 8w + 4u + l/16, position l%16 (the hardware places the
   // lanes back to back) and therefore fetches chunk (l%16) ^ swz(row).  Rows past the end of the chunk
   // are out of the descriptor's range and arrive as zeros.
-  auto swz = [](int row) { return ((row & 3) << 2) | ((row >> 2) & 3); };
+  auto swz = [](int row) { return lds_row_swizzle(row); };
   const u32x4 krs = rsrc_words(p.k + b * p.k_sb + hk * p.k_sh, (uint32_t)(((int64_t)(p.Sc - 1) * p.k_ss + kD) * 2));
   const u32x4 vrs = rsrc_words(p.v + b * p.v_sb + hk * p.v_sh, (uint32_t)(((int64_t)(p.Sc - 1) * p.v_ss + kD) * 2));
   int kvoff[2], vvoff[2];

@@ -56,6 +56,41 @@ __device__ __forceinline__ float pair_sum(float x) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
+// Buffer descriptor over `bytes` bytes at `base`, as four scalar words: loads whose offset (vector +
+// scalar part) falls past the end return zero.
+__device__ __forceinline__ u32x4 rsrc_words(const void* base, uint32_t bytes) {
+  const uint64_t a = (uint64_t)base;
+  u32x4 r;
+  // wavefront-uniform by construction; readfirstlane makes that visible to the register allocator
+  r[0] = __builtin_amdgcn_readfirstlane((uint32_t)a);
+  r[1] = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu);
+  r[2] = __builtin_amdgcn_readfirstlane(bytes);
+  r[3] = 0x00020000u;
+  return r;
+}
+
+// Global -> LDS copy of 16 (or 4) bytes per lane without passing through registers: lane l's bytes land
+// at LDS address `lds_addr` + 16 l (+ 4 l); the base is wavefront-uniform and travels in M0.  Lanes whose
+// offset is out of the descriptor's range write zeros.  Completion is counted by vmcnt.  Written as
+// inline assembly so that the compiler's own wait-count insertion does not see the copies: it would
+// otherwise wait for all of them before every transposing LDS read.  The kernels place the waits by hand.
+__device__ __forceinline__ void copy16_to_lds(u32x4 rsrc, uint32_t lds_addr, int voffset, int soffset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voffset), "s"(rsrc),
+                  "s"(__builtin_amdgcn_readfirstlane(soffset)) : "memory");
+}
+__device__ __forceinline__ void copy4_to_lds(u32x4 rsrc, uint32_t lds_addr, int voffset, int soffset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+               :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voffset), "s"(rsrc),
+                  "s"(__builtin_amdgcn_readfirstlane(soffset)) : "memory");
+}
+
+// Tiles copied that way are rows of 256 bytes (128 bf16) without padding; chunk c (16 bytes) of row r is
+// kept at chunk position c ^ lds_row_swizzle(r).  With this map both access patterns of the MFMA operand
+// reads are free of bank conflicts: 32 consecutive rows x one chunk (ds_read_b128 of a row-major operand)
+// and 8 rows x 4 consecutive chunks (ds_read_b64_tr_b16 of a transposed operand).
+__device__ __forceinline__ constexpr int lds_row_swizzle(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 inline int launch_status() {
