@@ -138,7 +138,7 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
       yf[ks] = *reinterpret_cast<const bf16x8*>(yp + ks * 16);
     }
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) { asm volatile("" : "+v"(xf[ks])); asm volatile("" : "+v"(yf[ks])); }
+    for (int ks = 0; ks < 8; ++ks) { asm volatile("" : "+a"(xf[ks])); asm volatile("" : "+a"(yf[ks])); }
   }
   // DQ: the query is the stationary row, its lse2 / delta are per-lane scalars
   float lse2_lane = 0.f, delta_lane = 0.f;
@@ -239,13 +239,6 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
       }
   }
   typedef __attribute__((address_space(3))) bf16x4* lds_bf16x4;
-  auto read_tr = [&](const unsigned char* tile, int db, int kstep) -> bf16x8 {
-    const unsigned char* base = tile + (kstep >> 1) * 8192 + (kstep & 1) * 4096;
-    const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4)(base + tr_rd[db][0]));
-    const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4)(base + tr_rd[db][1]));
-    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-  };
-
   f32x16 acc1[4], acc2[4];      // DQ: acc1 = dQ^T.  Otherwise acc1 = dK^T, acc2 = dV^T
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -253,103 +246,101 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     for (int j = 0; j < 16; ++j) { acc1[i][j] = 0.f; acc2[i][j] = 0.f; }
   const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-  // Tile t lives in stage t % 4.  One step works on two tiles: the 32 MFMAs of T1 / T2 of tile t+1 are
-  // issued interleaved with the exponentials of tile t (whose T1 / T2 the step before left in registers),
-  // then the MFMAs that accumulate tile t follow.  A step starts by waiting for this wavefront's copies
-  // of tile t+1 (those of tile t+2 stay in flight) and a barrier: after it tile t+1 is complete for every
-  // wavefront and nobody reads tile t-1 any more, whose stage then receives tile t+3.  Tiles past the end
-  // are copied as zeros (and their T1 / T2 computed, unused) so that the number of copies in flight
-  // stays the same.
+  // Tile t lives in stage t % 4 and is processed as two halves of 32 streamed rows.  One half-step issues
+  // the 16 MFMAs of T1 / T2 of the NEXT half interleaved with the exponentials of the current half (whose
+  // T1 / T2 the half-step before left in registers), then the MFMAs that accumulate the current half.
+  // The second half-step of tile t is the one that reaches into tile t+1: it starts by waiting for this
+  // wavefront's copies of tile t+1 (those of tile t+2 stay in flight) and a barrier, after which tile t+1 is
+  // complete for every wavefront and nobody reads tile t-1 any more, whose stage then receives tile t+3.
+  // Tiles past the end are copied as zeros (and their T1 / T2 computed, unused) so that the number of
+  // copies in flight stays the same.
   constexpr int kDepth = 4;                                // operand reads in flight ahead of the MFMAs
-  auto read_rm = [&](const unsigned char* xs, int i) -> bf16x8 {        // slot i of the T1 / T2 sequence
-    const int kk = i >> 2, mb = (i >> 1) & 1;
-    return *reinterpret_cast<const bf16x8*>(xs + ((i & 1) ? kOffY : 0) + rm_rd[kk] + mb * 8192);
+  typedef __attribute__((address_space(3))) const bf16x8* lds_bf16x8;
+  typedef __attribute__((address_space(3))) const f32x4* lds_f32x4;
+  // slot i (0..15) of the T1 / T2 sequence of one half: k-step i / 2, X (T1) on even and Y (T2) on odd slots
+  auto read_rm = [&](const int (&rm)[8], int mb, int i) -> bf16x8 {
+    return *(lds_bf16x8)(uintptr_t)(uint32_t)(rm[i >> 1] + mb * 8192 + ((i & 1) ? kOffY : 0));
   };
-  auto t_mfma = [&](int i, const bf16x8& a, f32x16 (&n1)[2], f32x16 (&n2)[2]) {
-    const int kk = i >> 2, mb = (i >> 1) & 1;
-    if (i & 1) n2[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, yf[kk], kk == 0 ? zero : n2[mb], 0, 0, 0);
-    else n1[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, xf[kk], kk == 0 ? zero : n1[mb], 0, 0, 0);
+  auto t_mfma = [&](int i, const bf16x8& a, f32x16& n1, f32x16& n2) {
+    const int kk = i >> 1;
+    if (i & 1) n2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, yf[kk], kk == 0 ? zero : n2, 0, 0, 0);
+    else n1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, xf[kk], kk == 0 ? zero : n1, 0, 0, 0);
   };
-  // T1 / T2 of one tile without anything interleaved (first tile)
-  auto t_only = [&](int stage, f32x16 (&n1)[2], f32x16 (&n2)[2]) {
-    const unsigned char* xs = smem + stage * kStageBytes;
-    bf16x8 ring[kDepth];
+  // LDS byte addresses of the operand reads for the tile in `stage`
+  auto tile_addrs = [&](int stage, int (&rm)[8], int (&tr)[4][2]) {
+    const int base = (int)lds_base + stage * kStageBytes;
 #pragma unroll
-    for (int i = 0; i < kDepth; ++i) ring[i] = read_rm(xs, i);
+    for (int kk = 0; kk < 8; ++kk) rm[kk] = rm_rd[kk] + base;
 #pragma unroll
-    for (int i = 0; i < 32; ++i) {
-      t_mfma(i, ring[i % kDepth], n1, n2);
-      if (i + kDepth < 32) ring[i % kDepth] = read_rm(xs, i + kDepth);
-    }
+    for (int db = 0; db < 4; ++db) { tr[db][0] = tr_rd[db][0] + base; tr[db][1] = tr_rd[db][1] + base; }
   };
-  bf16x8 pfrag[4], dsfrag[4];
-  // P and dS of element j (accumulator register) of block mb of the current tile, in place
-  auto p_ds = [&](int mb, int j, const f32x4& lv, const f32x4& dv, f32x16 (&c1)[2], f32x16 (&c2)[2],
-                  bool need_mask, int c0) {
-    const int g = j >> 2, e = j & 3;
-    const float l = DQ ? lse2_lane : lv[e];
-    const float d = DQ ? delta_lane : dv[e];
-    float pe = fast_exp2(__builtin_fmaf(c1[mb][j], p.scale_log2, -l));
+  auto read_tr_at = [&](const int (&tr)[4][2], int db, int kstep, bool y) -> bf16x8 {
+    const int off = (kstep >> 1) * 8192 + (kstep & 1) * 4096 + (y ? kOffY : 0);
+    const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4)(uintptr_t)(uint32_t)(tr[db][0] + off));
+    const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4)(uintptr_t)(uint32_t)(tr[db][1] + off));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+
+  bf16x8 pfrag[2], dsfrag[2];     // P and dS of the current half as B operands (two k-steps of 16 rows)
+  // Current half = block mb of the tile at (rm_c, tr_c), scores / dP in (c1, c2); next half = block nmb of
+  // the tile at rm_n, results into (n1, n2).
+  auto half_step = [&](int mb, int nmb, const int (&rm_c)[8], const int (&tr_c)[4][2], const int (&rm_n)[8],
+                       f32x16& c1, f32x16& c2, f32x16& n1, f32x16& n2, int c0, int stage_c) {
+    // Hidden elements of the current half (rows past the end of the streamed tensor, the causal mask) get
+    // a score of -inf, hence P = dS = 0.  Only the last tile of a head and the tiles the diagonal crosses
+    // need it.
+    const int cb = c0 + mb * 32;
+    bool need_mask = cb + 32 > n_str;
+    if (CAUSAL) need_mask = need_mask || (DQ ? (cb + 31 > r0 + shift) : (r0 + kRowsPerWg - 1 > cb + shift));
     if (need_mask) {
-      const int c = c0 + mb * 32 + g * 8 + hf * 4 + e;     // streamed row of this element
-      bool hidden = c >= n_str;
-      if (CAUSAL) hidden = hidden || (DQ ? (c > my_r + shift) : (my_r > c + shift));
-      if (hidden) pe = 0.f;
-    }
-    c1[mb][j] = pe;
-    c2[mb][j] = pe * (c2[mb][j] - d);
-  };
-  auto pack_frags = [&](int mb, int j2, const f32x16 (&c1)[2], const f32x16 (&c2)[2]) {
-    u32x4 wp, wd;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      wp[e] = pack_bf16(c1[mb][8 * j2 + 2 * e], c1[mb][8 * j2 + 2 * e + 1]);
-      wd[e] = pack_bf16(c2[mb][8 * j2 + 2 * e], c2[mb][8 * j2 + 2 * e + 1]);
+      for (int j = 0; j < 16; ++j) {
+        const int c = cb + (j >> 2) * 8 + hf * 4 + (j & 3);     // streamed row of this element
+        bool hidden = c >= n_str;
+        if (CAUSAL) hidden = hidden || (DQ ? (c > my_r + shift) : (my_r > c + shift));
+        if (hidden) c1[j] = -INFINITY;
+      }
     }
-    pfrag[mb * 2 + j2] = __builtin_bit_cast(bf16x8, wp);
-    dsfrag[mb * 2 + j2] = __builtin_bit_cast(bf16x8, wd);
-  };
-
-  auto step = [&](int t, f32x16 (&c1)[2], f32x16 (&c2)[2], f32x16 (&n1)[2], f32x16 (&n2)[2]) {
-    if (DQ) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
-    static_assert(kCopiesPerTile == (DQ ? 8 : 9), "the vmcnt immediates are one tile of copies");
-    __builtin_amdgcn_s_barrier();
-    copy_tile(t + 3, (t + 3) & 3);
-    const unsigned char* xs = smem + (t & 3) * kStageBytes;            // tile t
-    const unsigned char* xn = smem + ((t + 1) & 3) * kStageBytes;      // tile t+1
-    const int c0 = tile_row0(t);
-    bool need_mask = c0 + kTile > n_str;                       // rows past the end of the streamed tensor
-    if (CAUSAL) need_mask = need_mask || (DQ ? (c0 + kTile - 1 > r0 + shift) : (r0 + kRowsPerWg - 1 > c0 + shift));
-
-    // ---- T1 / T2 of tile t+1 (slot i = one MFMA), P / dS of tile t (slot i = element i % 16 of block i / 16) ----
+    // ---- T1 / T2 of the next half (slot i = one MFMA), P / dS of the current half (slot i = register i) ----
     {
       bf16x8 ring[kDepth];
 #pragma unroll
-      for (int i = 0; i < kDepth; ++i) ring[i] = read_rm(xn, i);
+      for (int i = 0; i < kDepth; ++i) ring[i] = read_rm(rm_n, nmb, i);
       f32x4 lv = {0.f, 0.f, 0.f, 0.f}, dv = {0.f, 0.f, 0.f, 0.f};
+      const int ld_addr = (int)lds_base + stage_c * kStageBytes + kOffLse + (mb * 32 + hf * 4) * 4;
 #pragma unroll
-      for (int i = 0; i < 32; ++i) {
+      for (int i = 0; i < 16; ++i) {
         t_mfma(i, ring[i % kDepth], n1, n2);
-        if (i + kDepth < 32) ring[i % kDepth] = read_rm(xn, i + kDepth);
-        const int mb = i >> 4, j = i & 15;
-        if (!DQ && (j & 3) == 0) {
-          const int row = mb * 32 + (j >> 2) * 8 + hf * 4;
-          lv = *reinterpret_cast<const f32x4*>(xs + kOffLse + row * 4);
-          dv = *reinterpret_cast<const f32x4*>(xs + kOffDelta + row * 4);
+        if (i + kDepth < 16) ring[i % kDepth] = read_rm(rm_n, nmb, i + kDepth);
+        if (!DQ && (i & 3) == 0) {
+          lv = *(lds_f32x4)(uintptr_t)(uint32_t)(ld_addr + (i >> 2) * 32);
+          dv = *(lds_f32x4)(uintptr_t)(uint32_t)(ld_addr + (i >> 2) * 32 + (kOffDelta - kOffLse));
         }
-        p_ds(mb, j, lv, dv, c1, c2, need_mask, c0);
-        if ((j & 7) == 7) pack_frags(mb, j >> 3, c1, c2);
+        const float l = DQ ? lse2_lane : lv[i & 3];
+        const float d = DQ ? delta_lane : dv[i & 3];
+        const float pe = fast_exp2(__builtin_fmaf(c1[i], p.scale_log2, -l));
+        c1[i] = pe;
+        c2[i] = pe * (c2[i] - d);
+        if ((i & 7) == 7) {
+          const int j2 = i >> 3;
+          u32x4 wp, wd;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            wp[e] = pack_bf16(c1[8 * j2 + 2 * e], c1[8 * j2 + 2 * e + 1]);
+            wd[e] = pack_bf16(c2[8 * j2 + 2 * e], c2[8 * j2 + 2 * e + 1]);
+          }
+          pfrag[j2] = __builtin_bit_cast(bf16x8, wp);
+          dsfrag[j2] = __builtin_bit_cast(bf16x8, wd);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    // ---- acc1^T += X_str^T dS,  acc2^T += Y_str^T P  (tile t) ---------------------------------------------
+    // ---- acc1^T += X_str^T dS,  acc2^T += Y_str^T P  (current half: k-steps 2 mb, 2 mb + 1) ---------------
     {
-      constexpr int kN = DQ ? 16 : 32;
+      constexpr int kN = DQ ? 8 : 16;
       auto read_acc = [&](int i) -> bf16x8 {
         const int m = DQ ? i : (i >> 1);
-        const int db = m & 3, kstep = m >> 2;
-        return read_tr((DQ || !(i & 1)) ? xs : xs + kOffY, db, kstep);
+        return read_tr_at(tr_c, m & 3, mb * 2 + (m >> 2), !DQ && (i & 1));
       };
       bf16x8 ring[kDepth];
 #pragma unroll
@@ -357,32 +348,51 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
 #pragma unroll
       for (int i = 0; i < kN; ++i) {
         const int m = DQ ? i : (i >> 1);
-        const int db = m & 3, kstep = m >> 2;
-        if (DQ || !(i & 1)) acc1[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % kDepth], dsfrag[kstep], acc1[db], 0, 0, 0);
-        else acc2[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % kDepth], pfrag[kstep], acc2[db], 0, 0, 0);
+        const int db = m & 3, j2 = m >> 2;
+        if (DQ || !(i & 1)) acc1[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % kDepth], dsfrag[j2], acc1[db], 0, 0, 0);
+        else acc2[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % kDepth], pfrag[j2], acc2[db], 0, 0, 0);
         if (i + kDepth < kN) ring[i % kDepth] = read_acc(i + kDepth);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
   };
 
-  f32x16 ta1[2], ta2[2], tb1[2], tb2[2];
+  f32x16 ta1, ta2, tb1, tb2;          // T1 / T2 of the two halves in flight
+  int rm_c[8], tr_c[4][2], rm_n[8], tr_n[4][2];
   if (ntiles > 0) {
     copy_tile(0, 0);
     copy_tile(1, 1);
     copy_tile(2, 2);
     if (DQ) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
+    static_assert(kCopiesPerTile == (DQ ? 8 : 9), "the vmcnt immediates are one and two tiles of copies");
     __builtin_amdgcn_s_barrier();
-    t_only(0, ta1, ta2);
-  }
-  {
-    int t = 0;
-    for (; t + 1 < ntiles; t += 2) {
-      step(t, ta1, ta2, tb1, tb2);
-      step(t + 1, tb1, tb2, ta1, ta2);
+    tile_addrs(0, rm_c, tr_c);
+    // T1 / T2 of the first half of tile 0, nothing to interleave with
+    bf16x8 ring[kDepth];
+#pragma unroll
+    for (int i = 0; i < kDepth; ++i) ring[i] = read_rm(rm_c, 0, i);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      t_mfma(i, ring[i % kDepth], ta1, ta2);
+      if (i + kDepth < 16) ring[i % kDepth] = read_rm(rm_c, 0, i + kDepth);
     }
-    if (t < ntiles) step(t, ta1, ta2, tb1, tb2);
+  }
+  for (int t = 0; t < ntiles; ++t) {
+    const int c0 = tile_row0(t);
+    // first half: next half is the second half of the same tile
+    half_step(0, 1, rm_c, tr_c, rm_c, ta1, ta2, tb1, tb2, c0, t & 3);
+    // second half: next half is the first half of tile t+1
+    if (DQ) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    copy_tile(t + 3, (t + 3) & 3);
+    tile_addrs((t + 1) & 3, rm_n, tr_n);
+    half_step(1, 0, rm_c, tr_c, rm_n, tb1, tb2, ta1, ta2, c0, t & 3);
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) rm_c[kk] = rm_n[kk];
+#pragma unroll
+    for (int db = 0; db < 4; ++db) { tr_c[db][0] = tr_n[db][0]; tr_c[db][1] = tr_n[db][1]; }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the zero-filled copies of tiles past the end
 

@@ -17,6 +17,12 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
+# attn_bwd.hip keeps 128 accumulator registers per lane for dK^T / dV^T and works on T1 / T2 with the vector
+# unit: with MFMA results in arithmetic registers (and only the stationary operands in accumulation
+# registers) there are no copies between the two register files in its main loop.
+EXTRA_FLAGS = {"attn_bwd.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
+
 def _run(cmd):
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
@@ -28,7 +34,8 @@ def _run(cmd):
 def build(verbose: bool = False) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objs = [os.path.join(HERE, s.replace(".hip", ".o")) for s in SOURCES]
-    cmds = [[hipcc, *FLAGS, "-c", os.path.join(HERE, s), "-o", o] for s, o in zip(SOURCES, objs)]
+    cmds = [[hipcc, *FLAGS, *EXTRA_FLAGS.get(s, []), "-c", os.path.join(HERE, s), "-o", o]
+            for s, o in zip(SOURCES, objs)]
     with ThreadPoolExecutor(max_workers=min(4, len(cmds))) as ex:
         for out in ex.map(_run, cmds):
             if verbose and out.strip():
