@@ -246,15 +246,21 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     for (int j = 0; j < 16; ++j) { acc1[i][j] = 0.f; acc2[i][j] = 0.f; }
   const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-  // Tile t lives in stage t % 4 and is processed as two halves of 32 streamed rows.  One half-step issues
-  // the 16 MFMAs of T1 / T2 of the NEXT half interleaved with the exponentials of the current half (whose
-  // T1 / T2 the half-step before left in registers), then the MFMAs that accumulate the current half.
-  // The second half-step of tile t is the one that reaches into tile t+1: it starts by waiting for this
-  // wavefront's copies of tile t+1 (those of tile t+2 stay in flight) and a barrier, after which tile t+1 is
-  // complete for every wavefront and nobody reads tile t-1 any more, whose stage then receives tile t+3.
-  // Tiles past the end are copied as zeros (and their T1 / T2 computed, unused) so that the number of
-  // copies in flight stays the same.
+  // Tile t lives in stage t % 4 and is processed as two halves of 32 streamed rows.  Per tile the matrix
+  // pipe sees one unbroken sequence of MFMA slots in four phases:
+  //   P0  T1 / T2 of (t, second half)      16 slots, each carrying P / dS of one register of (t, first half)
+  //   P1  accumulate (t, first half)       16 slots (8 for dQ)
+  //   P2  T1 / T2 of (t+1, first half)     16 slots, each carrying P / dS of one register of (t, second half)
+  //   P3  accumulate (t, second half)      16 slots (8 for dQ)
+  // The LDS operand of slot s+4 is read in slot s, across phase and tile boundaries, so the pipe never
+  // waits for LDS at the start of a phase.  An iteration starts by waiting for this wavefront's copies of
+  // tile t+1 (those of tile t+2 stay in flight) and a barrier, after which tile t+1 is complete for every
+  // wavefront and nobody reads tile t-1 any more, whose stage then receives tile t+3.  Tiles past the end
+  // are copied as zeros (and their T1 / T2 computed, unused) so that the number of copies in flight
+  // stays the same.
   constexpr int kDepth = 4;                                // operand reads in flight ahead of the MFMAs
+  constexpr int kAcc = DQ ? 8 : 16;                        // slots of an accumulate phase
+  constexpr int kP1 = 16, kP2 = 16 + kAcc, kP3 = 32 + kAcc, kSlots = 32 + 2 * kAcc;
   typedef __attribute__((address_space(3))) const bf16x8* lds_bf16x8;
   typedef __attribute__((address_space(3))) const f32x4* lds_f32x4;
   // slot i (0..15) of the T1 / T2 sequence of one half: k-step i / 2, X (T1) on even and Y (T2) on odd slots
@@ -274,22 +280,24 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
 #pragma unroll
     for (int db = 0; db < 4; ++db) { tr[db][0] = tr_rd[db][0] + base; tr[db][1] = tr_rd[db][1] + base; }
   };
-  auto read_tr_at = [&](const int (&tr)[4][2], int db, int kstep, bool y) -> bf16x8 {
-    const int off = (kstep >> 1) * 8192 + (kstep & 1) * 4096 + (y ? kOffY : 0);
-    const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4)(uintptr_t)(uint32_t)(tr[db][0] + off));
-    const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4)(uintptr_t)(uint32_t)(tr[db][1] + off));
+  // slot i of an accumulate phase of half mb: head-dim block and k-step, X^T (dS) / Y^T (P) alternating for dK, dV
+  auto read_acc = [&](const int (&tr)[4][2], int mb, int i) -> bf16x8 {
+    const int m = DQ ? i : (i >> 1);
+    const int off = mb * 8192 + (m >> 2) * 4096 + ((!DQ && (i & 1)) ? kOffY : 0);
+    const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4)(uintptr_t)(uint32_t)(tr[m & 3][0] + off));
+    const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4)(uintptr_t)(uint32_t)(tr[m & 3][1] + off));
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   };
 
-  bf16x8 pfrag[2], dsfrag[2];     // P and dS of the current half as B operands (two k-steps of 16 rows)
-  // Current half = block mb of the tile at (rm_c, tr_c), scores / dP in (c1, c2); next half = block nmb of
-  // the tile at rm_n, results into (n1, n2).
-  auto half_step = [&](int mb, int nmb, const int (&rm_c)[8], const int (&tr_c)[4][2], const int (&rm_n)[8],
-                       f32x16& c1, f32x16& c2, f32x16& n1, f32x16& n2, int c0, int stage_c) {
-    // Hidden elements of the current half (rows past the end of the streamed tensor, the causal mask) get
-    // a score of -inf, hence P = dS = 0.  Only the last tile of a head and the tiles the diagonal crosses
-    // need it.
-    const int cb = c0 + mb * 32;
+  bf16x8 pfrag[2], dsfrag[2];     // P and dS of the half being accumulated as B operands (two k-steps)
+  bf16x8 ring[kDepth];
+  f32x16 ta1, ta2, tb1, tb2;      // T1 / T2 of the two halves in flight: (t, first half), (t, second half)
+  int rm_c[8], tr_c[4][2], rm_n[8], tr_n[4][2];
+  f32x4 lv[5], dv[5];             // lse2 / delta of 4 streamed rows per entry (dK / dV pass), read one group ahead
+
+  // Hidden elements (rows past the end of the streamed tensor, the causal mask) get a score of -inf,
+  // hence P = dS = 0.  Only the last tile of a head and the tiles the diagonal crosses need it.
+  auto mask_half = [&](f32x16& c1, int cb) {
     bool need_mask = cb + 32 > n_str;
     if (CAUSAL) need_mask = need_mask || (DQ ? (cb + 31 > r0 + shift) : (r0 + kRowsPerWg - 1 > cb + shift));
     if (need_mask) {
@@ -301,64 +309,48 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
         if (hidden) c1[j] = -INFINITY;
       }
     }
-    // ---- T1 / T2 of the next half (slot i = one MFMA), P / dS of the current half (slot i = register i) ----
-    {
-      bf16x8 ring[kDepth];
+  };
+  // lse2 / delta of rows 8 g + 4 hf .. + 3 of half mb of the tile in `stage`
+  auto read_ld = [&](int stage, int mb, int g, f32x4& l, f32x4& d) {
+    const int addr = (int)lds_base + stage * kStageBytes + kOffLse + (mb * 32 + g * 8 + hf * 4) * 4;
+    l = *(lds_f32x4)(uintptr_t)(uint32_t)addr;
+    d = *(lds_f32x4)(uintptr_t)(uint32_t)(addr + (kOffDelta - kOffLse));
+  };
+  // P / dS of accumulator register i of the half in (c1, c2), packed into B operands every 8 registers
+  auto vector_slot = [&](int i, f32x16& c1, f32x16& c2, int stage, int mb) {
+    if (!DQ && (i & 3) == 0 && i < 12) read_ld(stage, mb, (i >> 2) + 1, lv[(i >> 2) + 1], dv[(i >> 2) + 1]);
+    const float l = DQ ? lse2_lane : lv[i >> 2][i & 3];
+    const float d = DQ ? delta_lane : dv[i >> 2][i & 3];
+    const float pe = fast_exp2(__builtin_fmaf(c1[i], p.scale_log2, -l));
+    c1[i] = pe;
+    c2[i] = pe * (c2[i] - d);
+    if ((i & 7) == 7) {
+      const int j2 = i >> 3;
+      u32x4 wp, wd;
 #pragma unroll
-      for (int i = 0; i < kDepth; ++i) ring[i] = read_rm(rm_n, nmb, i);
-      f32x4 lv = {0.f, 0.f, 0.f, 0.f}, dv = {0.f, 0.f, 0.f, 0.f};
-      const int ld_addr = (int)lds_base + stage_c * kStageBytes + kOffLse + (mb * 32 + hf * 4) * 4;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        t_mfma(i, ring[i % kDepth], n1, n2);
-        if (i + kDepth < 16) ring[i % kDepth] = read_rm(rm_n, nmb, i + kDepth);
-        if (!DQ && (i & 3) == 0) {
-          lv = *(lds_f32x4)(uintptr_t)(uint32_t)(ld_addr + (i >> 2) * 32);
-          dv = *(lds_f32x4)(uintptr_t)(uint32_t)(ld_addr + (i >> 2) * 32 + (kOffDelta - kOffLse));
-        }
-        const float l = DQ ? lse2_lane : lv[i & 3];
-        const float d = DQ ? delta_lane : dv[i & 3];
-        const float pe = fast_exp2(__builtin_fmaf(c1[i], p.scale_log2, -l));
-        c1[i] = pe;
-        c2[i] = pe * (c2[i] - d);
-        if ((i & 7) == 7) {
-          const int j2 = i >> 3;
-          u32x4 wp, wd;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            wp[e] = pack_bf16(c1[8 * j2 + 2 * e], c1[8 * j2 + 2 * e + 1]);
-            wd[e] = pack_bf16(c2[8 * j2 + 2 * e], c2[8 * j2 + 2 * e + 1]);
-          }
-          pfrag[j2] = __builtin_bit_cast(bf16x8, wp);
-          dsfrag[j2] = __builtin_bit_cast(bf16x8, wd);
-        }
-        __builtin_amdgcn_sched_barrier(0);
+      for (int e = 0; e < 4; ++e) {
+        wp[e] = pack_bf16(c1[8 * j2 + 2 * e], c1[8 * j2 + 2 * e + 1]);
+        wd[e] = pack_bf16(c2[8 * j2 + 2 * e], c2[8 * j2 + 2 * e + 1]);
       }
-    }
-    // ---- acc1^T += X_str^T dS,  acc2^T += Y_str^T P  (current half: k-steps 2 mb, 2 mb + 1) ---------------
-    {
-      constexpr int kN = DQ ? 8 : 16;
-      auto read_acc = [&](int i) -> bf16x8 {
-        const int m = DQ ? i : (i >> 1);
-        return read_tr_at(tr_c, m & 3, mb * 2 + (m >> 2), !DQ && (i & 1));
-      };
-      bf16x8 ring[kDepth];
-#pragma unroll
-      for (int i = 0; i < kDepth; ++i) ring[i] = read_acc(i);
-#pragma unroll
-      for (int i = 0; i < kN; ++i) {
-        const int m = DQ ? i : (i >> 1);
-        const int db = m & 3, j2 = m >> 2;
-        if (DQ || !(i & 1)) acc1[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % kDepth], dsfrag[j2], acc1[db], 0, 0, 0);
-        else acc2[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[i % kDepth], pfrag[j2], acc2[db], 0, 0, 0);
-        if (i + kDepth < kN) ring[i % kDepth] = read_acc(i + kDepth);
-        __builtin_amdgcn_sched_barrier(0);
-      }
+      pfrag[j2] = __builtin_bit_cast(bf16x8, wp);
+      dsfrag[j2] = __builtin_bit_cast(bf16x8, wd);
     }
   };
+  auto acc_mfma = [&](int i, const bf16x8& a) {
+    const int m = DQ ? i : (i >> 1);
+    const int db = m & 3, j2 = m >> 2;
+    if (DQ || !(i & 1)) acc1[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, dsfrag[j2], acc1[db], 0, 0, 0);
+    else acc2[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pfrag[j2], acc2[db], 0, 0, 0);
+  };
+  // LDS operand of slot s of the current tile's sequence; s >= kSlots continues into the next tile's P0
+  auto read_slot = [&](int s) -> bf16x8 {
+    if (s >= kSlots) return read_rm(rm_n, 1, s - kSlots);
+    if (s < kP1) return read_rm(rm_c, 1, s);
+    if (s < kP2) return read_acc(tr_c, 0, s - kP1);
+    if (s < kP3) return read_rm(rm_n, 0, s - kP2);
+    return read_acc(tr_c, 1, s - kP3);
+  };
 
-  f32x16 ta1, ta2, tb1, tb2;          // T1 / T2 of the two halves in flight
-  int rm_c[8], tr_c[4][2], rm_n[8], tr_n[4][2];
   if (ntiles > 0) {
     copy_tile(0, 0);
     copy_tile(1, 1);
@@ -369,7 +361,6 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     __builtin_amdgcn_s_barrier();
     tile_addrs(0, rm_c, tr_c);
     // T1 / T2 of the first half of tile 0, nothing to interleave with
-    bf16x8 ring[kDepth];
 #pragma unroll
     for (int i = 0; i < kDepth; ++i) ring[i] = read_rm(rm_c, 0, i);
 #pragma unroll
@@ -377,18 +368,50 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
       t_mfma(i, ring[i % kDepth], ta1, ta2);
       if (i + kDepth < 16) ring[i % kDepth] = read_rm(rm_c, 0, i + kDepth);
     }
+#pragma unroll
+    for (int i = 0; i < kDepth; ++i) ring[i] = read_rm(rm_c, 1, i);      // slots 0 .. 3 of tile 0
+    if (!DQ) read_ld(0, 0, 0, lv[0], dv[0]);
   }
   for (int t = 0; t < ntiles; ++t) {
     const int c0 = tile_row0(t);
-    // first half: next half is the second half of the same tile
-    half_step(0, 1, rm_c, tr_c, rm_c, ta1, ta2, tb1, tb2, c0, t & 3);
-    // second half: next half is the first half of tile t+1
+    const int stage = t & 3;
     if (DQ) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     copy_tile(t + 3, (t + 3) & 3);
     tile_addrs((t + 1) & 3, rm_n, tr_n);
-    half_step(1, 0, rm_c, tr_c, rm_n, tb1, tb2, ta1, ta2, c0, t & 3);
+    static_assert(kP1 % kDepth == 0 && kP2 % kDepth == 0 && kP3 % kDepth == 0 && kSlots % kDepth == 0,
+                  "every phase starts at ring entry 0");
+    mask_half(ta1, c0);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {                       // P0
+      t_mfma(i, ring[i % kDepth], tb1, tb2);
+      vector_slot(i, ta1, ta2, stage, 0);
+      ring[i % kDepth] = read_slot(i + kDepth);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int i = 0; i < kAcc; ++i) {                     // P1
+      acc_mfma(i, ring[i % kDepth]);
+      if (!DQ && i == kAcc - 2) read_ld(stage, 1, 0, lv[0], dv[0]);
+      ring[i % kDepth] = read_slot(kP1 + i + kDepth);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    mask_half(tb1, c0 + 32);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {                       // P2
+      t_mfma(i, ring[i % kDepth], ta1, ta2);
+      vector_slot(i, tb1, tb2, stage, 1);
+      ring[i % kDepth] = read_slot(kP2 + i + kDepth);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int i = 0; i < kAcc; ++i) {                     // P3
+      acc_mfma(i, ring[i % kDepth]);
+      if (!DQ && i == kAcc - 2) read_ld((t + 1) & 3, 0, 0, lv[0], dv[0]);
+      ring[i % kDepth] = read_slot(kP3 + i + kDepth);
+      __builtin_amdgcn_sched_barrier(0);
+    }
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk) rm_c[kk] = rm_n[kk];
 #pragma unroll
