@@ -258,7 +258,10 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
   // wavefront and nobody reads tile t-1 any more, whose stage then receives tile t+3.  Tiles past the end
   // are copied as zeros (and their T1 / T2 computed, unused) so that the number of copies in flight
   // stays the same.
-  constexpr int kDepth = 4;                                // operand reads in flight ahead of the MFMAs
+#ifndef MHIP_BWD_DEPTH
+#define MHIP_BWD_DEPTH 4
+#endif
+  constexpr int kDepth = MHIP_BWD_DEPTH;                   // operand reads in flight ahead of the MFMAs
   constexpr int kAcc = DQ ? 8 : 16;                        // slots of an accumulate phase
   constexpr int kP1 = 16, kP2 = 16 + kAcc, kP3 = 32 + kAcc, kSlots = 32 + 2 * kAcc;
   typedef __attribute__((address_space(3))) const bf16x8* lds_bf16x8;
@@ -380,8 +383,7 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     __builtin_amdgcn_s_barrier();
     copy_tile(t + 3, (t + 3) & 3);
     tile_addrs((t + 1) & 3, rm_n, tr_n);
-    static_assert(kP1 % kDepth == 0 && kP2 % kDepth == 0 && kP3 % kDepth == 0 && kSlots % kDepth == 0,
-                  "every phase starts at ring entry 0");
+    static_assert(kSlots % kDepth == 0 && 16 % kDepth == 0, "the ring position is the slot number modulo its depth");
     mask_half(ta1, c0);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {                       // P0
@@ -392,24 +394,24 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     }
 #pragma unroll
     for (int i = 0; i < kAcc; ++i) {                     // P1
-      acc_mfma(i, ring[i % kDepth]);
+      acc_mfma(i, ring[(kP1 + i) % kDepth]);
       if (!DQ && i == kAcc - 2) read_ld(stage, 1, 0, lv[0], dv[0]);
-      ring[i % kDepth] = read_slot(kP1 + i + kDepth);
+      ring[(kP1 + i) % kDepth] = read_slot(kP1 + i + kDepth);
       __builtin_amdgcn_sched_barrier(0);
     }
     mask_half(tb1, c0 + 32);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {                       // P2
-      t_mfma(i, ring[i % kDepth], ta1, ta2);
+      t_mfma(i, ring[(kP2 + i) % kDepth], ta1, ta2);
       vector_slot(i, tb1, tb2, stage, 1);
-      ring[i % kDepth] = read_slot(kP2 + i + kDepth);
+      ring[(kP2 + i) % kDepth] = read_slot(kP2 + i + kDepth);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int i = 0; i < kAcc; ++i) {                     // P3
-      acc_mfma(i, ring[i % kDepth]);
+      acc_mfma(i, ring[(kP3 + i) % kDepth]);
       if (!DQ && i == kAcc - 2) read_ld((t + 1) & 3, 0, 0, lv[0], dv[0]);
-      ring[i % kDepth] = read_slot(kP3 + i + kDepth);
+      ring[(kP3 + i) % kDepth] = read_slot(kP3 + i + kDepth);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll

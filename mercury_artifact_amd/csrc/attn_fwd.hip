@@ -55,12 +55,6 @@ struct FwdParams {
   int heads_per_xcd; // (batch, head) pairs per XCD when they divide evenly, else 0
 };
 
-// Buffer descriptor over `bytes` bytes at `base`: loads past the end return zero, so rows beyond the
-// chunk need no address clamping (their scores are masked afterwards).
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
-}
-
 template <bool CAUSAL>
 __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdParams p) {
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kStages * kTileBytes];
