@@ -23,7 +23,7 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, each counter scaled
 # by its reading for the calibration launch at the end of main() (profiles/ring_step_config1_hbm_traffic.md)
 TRAFFIC_FWD_BYTES = 134.9e6
-TRAFFIC_MERGE_BYTES = 173.2e6
+TRAFFIC_MERGE_BYTES = 171.5e6
 
 
 def cpu_baseline(sample_heads: int, B: int, Sq: int, D: int, W: int):
@@ -47,12 +47,60 @@ def cpu_baseline(sample_heads: int, B: int, Sq: int, D: int, W: int):
                       f"matmul/logsumexp + merge), {dt:.1f} s"}
 
 
+def other_kernels(torch, M, dev):
+    """Block kernels of the other configurations at their per-rank shapes, HIP events over 10 launches each
+    (reported next to the headline, not part of it)."""
+    def timeit(fn, n=10, w=3):
+        for _ in range(w):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    out = {}
+    B, S, H, D = 1, 4096, 32, 128
+    scale = D ** -0.5
+    q = torch.randn(B, S, H, D, device=dev).bfloat16()
+    kv = torch.randn(2, B, S, H, D, device=dev).bfloat16()
+    do = torch.randn(B, S, H, D, device=dev).bfloat16()
+    o = torch.empty_like(q)
+    lse = torch.empty(B, H, S, dtype=torch.float32, device=dev)
+    unit = 2.0 * B * H * S * S * D            # one S x S x D product per head
+    ms = timeit(lambda: M.attn_fwd_block(q, kv[0], kv[1], scale, causal=True, out=o, lse=lse))
+    out["fwd_bf16_causal_4096x4096"] = {"ms": round(ms, 4), "tflops": round(unit / ms / 1e9, 1),
+                                        "flops": "4 B H Sq Sc D / 2"}
+    M.attn_fwd_block(q, kv[0], kv[1], scale, out=o, lse=lse)
+    dq, dkv = torch.empty_like(q), torch.empty_like(kv)
+    ms = timeit(lambda: M.attn_bwd_block(do, q, kv[0], kv[1], o, lse, dq, dkv[0], dkv[1], scale))
+    out["bwd_bf16_4096x4096"] = {"ms": round(ms, 4), "tflops": round(5 * unit / ms / 1e9, 1),
+                                 "tflops_executed": round(7 * unit / ms / 1e9, 1),
+                                 "flops": "10 B H Sq Sc D algorithmic; the two-pass kernel executes 14"}
+    del dq, dkv, do
+    S8 = 16384
+    q8, sq = M.quantize_e4m3(torch.randn(B, S8, H, D, device=dev))
+    k8, sk = M.quantize_e4m3(torch.randn(B, S8, H, D, device=dev))
+    v8, sv = M.quantize_e4m3(torch.randn(B, S8, H, D, device=dev))
+    o8 = torch.empty(B, S8, H, D, dtype=torch.bfloat16, device=dev)
+    l8 = torch.empty(B, H, S8, dtype=torch.float32, device=dev)
+    ms = timeit(lambda: M.attn_fwd_block(q8, k8, v8, scale, q_descale=sq, k_descale=sk, v_descale=sv, out=o8, lse=l8),
+                n=5, w=2)
+    out["fwd_e4m3_16384x16384"] = {"ms": round(ms, 4), "tflops": round(4.0 * B * H * S8 * S8 * D / ms / 1e9, 1),
+                                   "pct_of_fp8_mfma_peak": round(4.0 * B * H * S8 * S8 * D / ms / 1e9 / 50.0, 2)}
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--cpu-heads", type=int, default=32, help="heads in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--no-variants", action="store_true",
+                    help="skip the short timings of the causal, backward and fp8 block kernels")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one rank's step on ONE GPU (the ring is emulated by local buffer rotation); "
@@ -142,6 +190,8 @@ def main() -> int:
     torch.cuda.synchronize()
     del calib
 
+    variants = None if args.no_variants else other_kernels(torch, M, dev)
+
     props = torch.cuda.get_device_properties(0)
     result = {
         "metric": "per-rank ring-attn step TFLOP/s + % MFMA peak (bf16, d128, Q 4096 x 8 chunks)",
@@ -169,6 +219,8 @@ def main() -> int:
                            "traffic": TRAFFIC_MERGE_BYTES, "avg_launch_ms": round(merge_ms, 5), "launches": len(real_merges),
                            "bytes_per_launch": merge_bytes},
     }
+    if variants is not None:
+        result["other_kernels"] = variants
     if args.cpu_heads > 0:
         result["cpu_baseline"] = cpu_baseline(args.cpu_heads, B, Sq, D, W)
     else:
