@@ -183,6 +183,24 @@ def main() -> int:
     torch.cuda.synchronize()
     fused_ms = (time.perf_counter() - t0) / args.steps * 1e3
 
+    # the same step replayed as one HIP graph (one launch instead of ~25; identical kernels and results)
+    FI.attn_fwd_block, MG.merge_into = real_fwd, real_merge
+    graph_ms, graph_same = None, None
+    try:
+        graphed = M.GraphedStep(step)
+        eager_o, eager_lse = o.clone(), lse.clone()
+        o.zero_()
+        graphed.replay()
+        torch.cuda.synchronize()
+        graph_same = bool(torch.equal(o, eager_o) and torch.equal(lse, eager_lse))
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graphed.replay()
+        torch.cuda.synchronize()
+        graph_ms = round((time.perf_counter() - t0) / args.steps * 1e3, 4)
+    except RuntimeError as exc:      # reported, never fatal for the headline number
+        print(f"bench.py: graph replay skipped: {exc}", file=sys.stderr)
+
     # one plain streaming kernel of known size (reads 128 MiB of bf16, writes 256 MiB of fp32): the
     # calibration point for the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this script
     calib = torch.empty(64 * 1024 * 1024, dtype=torch.bfloat16, device=dev).normal_()
@@ -210,6 +228,7 @@ def main() -> int:
                                "of 4096 (single ring, rank 0), 8 block forwards + 7 LSE merges + epilogue",
                    "flops_per_step": flops_per_step, "pct_of_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
                    "fused_epilogue_ms_per_step": round(fused_ms, 4),
+                   "hip_graph_ms_per_step": graph_ms, "hip_graph_bit_identical": graph_same,
                    "device": props.gcnArchName, "cus": props.multi_processor_count},
         "roofline": {"bound": "mfma", "kernel": "attn_fwd_bf16_d128", "achieved": round(fwd_tflops, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(fwd_tflops / PEAK_BF16_TFLOPS, 4),

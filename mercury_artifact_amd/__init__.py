@@ -10,6 +10,7 @@ from __future__ import annotations
 from . import _native
 from .flash_attn_interface import (_flash_attn_backward, _flash_attn_forward, attn_bwd_block,
                                    attn_fwd_block)
+from .graph import GraphedStep
 from .merge import (_update_out_and_lse, flash_reduce, get_default_args, grad_accumulate, merge_into,
                     pack_block, update_out_and_lse)
 from .ring import (flash_attn_backward, flash_attn_expose_reduce, flash_attn_pack_kv,

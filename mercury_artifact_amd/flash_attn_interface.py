@@ -119,9 +119,10 @@ def _(q, k, v, dropout_p, softmax_scale, causal, window_size_left, window_size_r
 
 
 def attn_bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_scale, causal=False,
-                   deterministic=False, dq_acc: Optional[torch.Tensor] = None) -> None:
+                   deterministic=False, dq_acc: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Block backward through mhip_attn_bwd_block; writes every element of dq, dk, dv in place and, if
-    ``dq_acc`` (fp32, contiguous, q's shape) is given, also adds the block's dq into it."""
+    ``dq_acc`` (fp32, contiguous, q's shape) is given, also adds the block's dq into it.  Returns
+    delta = rowsum(dout * out) as the kernel computed it, (B, Hq, Sq) fp32."""
     _check_block_inputs(q, k, v, 0, -1, -1, 0.0, None)
     N.require_cuda(dout, out, softmax_lse, dq, dk, dv, dq_acc)
     B, Sq, Hq, D = q.shape
@@ -164,6 +165,8 @@ def attn_bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_scale, c
     if dk_w is not dk:
         dk.copy_(dk_w)
         dv.copy_(dv_w)
+    # the workspace starts with delta = rowsum(dout * out), (B, Hq, Sq) fp32
+    return ws[: B * Hq * Sq * 4].view(torch.float32).view(B, Hq, Sq)
 
 
 @torch.library.custom_op("mercury_amd::_flash_attn_backward", mutates_args=("dq", "dk", "dv"),
@@ -192,6 +195,5 @@ def _flash_attn_backward(
     (``torch.empty``, utils/attn_bwd_dsl.py:83-84) and every element of them is written.
     Returns ``softmax_d`` (rowsum(dout * out), (B,Hq,Sq) fp32) like flash-attn does."""
     _check_block_inputs(q, k, v, dropout_p, window_size_left, window_size_right, softcap, alibi_slopes)
-    attn_bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_scale, bool(causal),
-                   bool(deterministic))
-    return (dout.float() * out.float()).sum(-1).transpose(1, 2).contiguous()
+    return attn_bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_scale, bool(causal),
+                          bool(deterministic)).clone()

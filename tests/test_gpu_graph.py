@@ -1,0 +1,70 @@
+"""A ring step replayed as a HIP graph gives, on every replay, exactly what the eager step gives.
+
+Replays are interleaved with eager work and synchronisations, and the inputs change in place between them:
+a graph that had frozen stale values, or whose nodes misbehave after the first replay, would fail."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_graphed_single_ring_step_matches_eager(fused):
+    import mercury_artifact_amd as M
+
+    B, S, H, D, W, rank = 2, 256, 4, 128, 4, 1
+    scale = D ** -0.5
+    g = torch.Generator(device="cuda").manual_seed(3)
+    q = torch.randn(B, S, H, D, generator=g, device="cuda").bfloat16()
+    chunks = [torch.randn(2, B, S, H, D, generator=g, device="cuda").bfloat16() for _ in range(W)]
+    o = torch.empty_like(q)
+    lse = torch.empty(B, H, S, dtype=torch.float32, device="cuda")
+
+    def step():
+        M.flash_attn_pack_kv(q, chunks[rank], o, lse, scale, ring=M.LocalRing((W,), rank, chunks),
+                             fused_epilogue=fused)
+
+    graphed = M.GraphedStep(step)
+    for it in range(4):
+        # new inputs, in place
+        q.copy_(torch.randn(B, S, H, D, generator=g, device="cuda").bfloat16())
+        chunks[(it + 1) % W].copy_(torch.randn(2, B, S, H, D, generator=g, device="cuda").bfloat16())
+        step()
+        torch.cuda.synchronize()
+        eo, el = o.clone(), lse.clone()
+        o.zero_()
+        lse.zero_()
+        (q.float() @ q.float().transpose(-1, -2)).sum().item()      # unrelated eager work + a sync
+        graphed.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(o, eo), it
+        assert torch.equal(lse, el), it
+
+
+def test_graphed_backward_block_matches_eager():
+    import mercury_artifact_amd as M
+
+    B, S, H, D = 1, 320, 2, 128
+    scale = D ** -0.5
+    g = torch.Generator(device="cuda").manual_seed(4)
+    q = torch.randn(B, S, H, D, generator=g, device="cuda").bfloat16()
+    kv = torch.randn(2, B, S, H, D, generator=g, device="cuda").bfloat16()
+    do = torch.randn(B, S, H, D, generator=g, device="cuda").bfloat16()
+    o, lse = M.attn_fwd_block(q, kv[0], kv[1], scale, causal=True)
+    dq, dkv = torch.empty_like(q), torch.empty_like(kv)
+
+    def step():
+        M.attn_bwd_block(do, q, kv[0], kv[1], o, lse, dq, dkv[0], dkv[1], scale, causal=True)
+
+    graphed = M.GraphedStep(step)
+    for it in range(3):
+        do.copy_(torch.randn(B, S, H, D, generator=g, device="cuda").bfloat16())
+        step()
+        torch.cuda.synchronize()
+        edq, edkv = dq.clone(), dkv.clone()
+        dq.zero_()
+        dkv.zero_()
+        torch.cuda.synchronize()
+        graphed.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(dq, edq) and torch.equal(dkv, edkv), it
