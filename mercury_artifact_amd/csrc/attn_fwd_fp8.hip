@@ -1,13 +1,18 @@
 // Block forward on e4m3 (OCP float8) Q/K/V for gfx950: out = softmax(scale * q k^T) v in bf16 and
-// lse in fp32, with x ~ descale_x * x_q per tensor.  fp8 MFMA (v_mfma_f32_32x32x16_fp8_fp8) for both
-// contractions, fp32 softmax.  Not in the reference; same call boundary as the bf16 kernel
-// (utils/flash_attn_dsl.py:159-176) with three extra descale arguments.
+// lse in fp32, with x ~ descale_x * x_q per tensor.  Both contractions run on the 64-deep fp8 MFMA
+// (v_mfma_f32_32x32x64_f8f6f4, twice the rate of the bf16 one), fp32 softmax.  Not in the reference; same
+// call boundary as the bf16 kernel (utils/flash_attn_dsl.py:159-176) with three extra descale arguments.
 //
-// Same decomposition as the bf16 kernel: 8 wavefronts x 32 Q rows per workgroup, wavefronts 0-3 stage K
-// and 4-7 stage V^T, S^T = K Q^T keeps one Q row per lane, P^T feeds the second MFMA from the
-// accumulator registers.  Differences:
-//   * a main-loop tile is 128 keys (the tile is as many bytes as the 64-key bf16 tile);
-//   * one 16-byte LDS read carries the A operands of two MFMA k-steps (8 fp8 values each);
+// Same decomposition as the bf16 kernel: 8 wavefronts x 32 Q rows per workgroup, S^T = K Q^T keeps one Q
+// row per lane, P^T feeds the second MFMA from the accumulator registers, K and V tiles are copied
+// global -> LDS without registers in between, four stages deep.  Differences:
+//   * a main-loop tile is 128 keys (as many bytes as the 64-key bf16 tile), rows of 128 bytes whose eight
+//     16-byte chunks are XOR-swizzled;
+//   * an MFMA takes 32 bytes per lane and operand: for S^T two 16-byte LDS reads of one K row, for O^T four
+//     ds_read_b64_tr_b8 of the row-major V tile (8 keys of one head-dim column each);
+//   * the K rows of a 32-key block are assigned to the MFMA rows through a permutation chosen so that a
+//     lane's 16 accumulator registers hold 16 CONSECUTIVE keys (16 hf + i): the transposing reads, which
+//     deliver 8 consecutive keys, then produce V^T in exactly the key order of the P registers;
 //   * the descales fold into the softmax scale (q, k) and the final normalisation (v);
 //   * P is multiplied by 2^7 before it is rounded to e4m3 (and the result divided by 2^7), so that small
 //     probabilities keep their relative precision; the reference score only lags the running maximum by
@@ -17,13 +22,16 @@
 namespace mhip {
 namespace {
 
+typedef __attribute__((__vector_size__(8 * sizeof(int)))) int i32x8;
+typedef __attribute__((__vector_size__(2 * sizeof(int)))) int i32x2;
+
 constexpr int kD = 128;
 constexpr int kWaves = 8;
 constexpr int kBM = kWaves * 32;
 constexpr int kBN = 128;              // keys per tile
-constexpr int kStride = 128 + 16;     // bytes per LDS row of K (128 head-dim bytes) and of V^T (128 keys)
-constexpr int kTileBytes = 128 * kStride;          // 18432, K and V^T alike
-constexpr int kStageBytes = 2 * kTileBytes;
+constexpr int kTileBytes = kBN * kD;  // 16384: one K or V tile in LDS, 128 rows of 128 bytes
+constexpr int kStages = 4;
+constexpr int kVBase = kStages * kTileBytes;
 constexpr int kOStride = kD + 8;
 constexpr float kPShift = 7.f;        // P is stored as 2^7 P in e4m3
 constexpr float kRescaleSlack = 1.f;
@@ -39,17 +47,14 @@ struct Fp8Params {
   int nq_tiles, total, per_xcd, heads_per_xcd;
 };
 
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
-}
-
-__device__ __forceinline__ long as_long(uint32_t lo, uint32_t hi) {
-  return (long)(((unsigned long)hi << 32) | lo);
-}
+// Chunk c (16 bytes) of row r of a tile lives at chunk position c ^ swz8(r).  Row pairs share a 256-byte
+// bank line, so the position inside the line is (r & 1, c ^ swz8(r)): the 32 rows of one 16-byte operand
+// read and the 16 rows x 2 chunks of one transposing read both cover the 16 positions exactly twice.
+__device__ __forceinline__ constexpr int swz8(int row) { return (((row >> 1) & 3) << 1) | ((row >> 3) & 1); }
 
 template <bool CAUSAL>
 __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Params p) {
-  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kStageBytes];
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kStages * kTileBytes];
 
   // Workgroup i runs on XCD i % 8: every XCD gets a contiguous range of (batch, head) pairs, so the
   // workgroups that share a K/V head share an L2.  Causal launches run the longest Q tiles first,
@@ -80,7 +85,6 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
   const int lane = tid & 63;
   const int ln = lane & 31;
   const int hf = lane >> 5;
-  const bool v_loader = wave >= 4;
 
   int kv_end = p.Sc;
   if (CAUSAL) {
@@ -90,78 +94,91 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
   }
   const int ntiles = (kv_end + kBN - 1) / kBN;
 
-  // ---- Q fragment: lane (ln, hf) holds bytes [32 i + 16 hf, +16) of its row; the first 8 are the B
-  // operand of k-step 2i, the last 8 of k-step 2i+1 (K is read from LDS with the same split) ------------
+  // ---- Q fragment: B operand of S^T, lane (ln, hf) holds bytes [64 ks + 32 hf, +32) of its row ------------
   const int my_q = q0 + wave * 32 + ln;
-  u32x4 qf[4];
+  i32x8 qf[2];
   {
     const int row = my_q < p.Sq ? my_q : p.Sq - 1;
-    const uint8_t* qp = p.q + b * p.q_sb + (int64_t)row * p.q_ss + hq * p.q_sh + hf * 16;
+    const uint8_t* qp = p.q + b * p.q_sb + (int64_t)row * p.q_ss + hq * p.q_sh + hf * 32;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) qf[i] = *reinterpret_cast<const u32x4*>(qp + i * 32);
+    for (int ks = 0; ks < 2; ++ks) {
+      const u32x4 lo = *reinterpret_cast<const u32x4*>(qp + ks * 64);
+      const u32x4 hi = *reinterpret_cast<const u32x4*>(qp + ks * 64 + 16);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(qf[i]));
-  }
-
-  // ---- staging: K loader thread lt loads rows (lt/8 + 32 i), 16-byte chunk lt%8; V loader thread loads
-  // the four rows of key quad lt/8, chunk lt%8 (16 head-dim values each) ---------------------------------
-  const int lt = tid & 255;
-  const int ld_chunk = lt & 7;
-  const int ld_row = lt >> 3;                        // 0..31
-  const uint8_t* gbase = v_loader ? p.v + b * p.v_sb + hk * p.v_sh : p.k + b * p.k_sb + hk * p.k_sh;
-  const int64_t g_ss = v_loader ? p.v_ss : p.k_ss;
-  const __amdgpu_buffer_rsrc_t grs = make_rsrc(gbase, (uint32_t)((int64_t)(p.Sc - 1) * g_ss + kD));
-  int goff[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-    goff[i] = (int)((v_loader ? ld_row * 4 + i : ld_row + 32 * i) * g_ss) + ld_chunk * 16;
-  const int tile_bytes = (int)(kBN * g_ss);
-  u32x4 greg[4];
-  auto load_tile = [&](int t) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) greg[i] = __builtin_amdgcn_raw_buffer_load_b128(grs, goff[i], t * tile_bytes, 0);
-  };
-
-  // V^T row d lives in LDS row d ^ ((d >> 4) & 7); inside a row, key quad (4 keys) u = 4-key index:
-  // 32-key block mb = u / 8, then (jj, thi, hf) = bits 2, 1, 0 of u % 8 -> byte (2 mb + hf) 16 + 8 jj + 4 thi,
-  // which is the order the accumulator registers of S^T hold the keys of two consecutive MFMA k-steps.
-  const int vt_off = ((ld_row >> 3) * 2 + (ld_row & 1)) * 16 + ((ld_row >> 2) & 1) * 8 + ((ld_row >> 1) & 1) * 4;
-  auto store_tile = [&](int stage) {
-    if (!v_loader) {
-      unsigned char* ks = smem + stage * kStageBytes;
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        *reinterpret_cast<u32x4*>(ks + (ld_row + 32 * i) * kStride + ld_chunk * 16) = greg[i];
-    } else {
-      unsigned char* vs = smem + stage * kStageBytes + kTileBytes;
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        // dword w of each of the four rows holds head-dim values 4w .. 4w+3 of this chunk
-        const uint32_t t01_lo = __builtin_amdgcn_perm(greg[1][w], greg[0][w], 0x05010400u);   // d0:(k0,k1) d1:(k0,k1)
-        const uint32_t t01_hi = __builtin_amdgcn_perm(greg[1][w], greg[0][w], 0x07030602u);   // d2, d3
-        const uint32_t t23_lo = __builtin_amdgcn_perm(greg[3][w], greg[2][w], 0x05010400u);
-        const uint32_t t23_hi = __builtin_amdgcn_perm(greg[3][w], greg[2][w], 0x07030602u);
-        uint32_t o[4];
-        o[0] = __builtin_amdgcn_perm(t23_lo, t01_lo, 0x05040100u);
-        o[1] = __builtin_amdgcn_perm(t23_lo, t01_lo, 0x07060302u);
-        o[2] = __builtin_amdgcn_perm(t23_hi, t01_hi, 0x05040100u);
-        o[3] = __builtin_amdgcn_perm(t23_hi, t01_hi, 0x07060302u);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int d = ld_chunk * 16 + ((4 * w + e) ^ ld_chunk);
-          *reinterpret_cast<uint32_t*>(vs + d * kStride + vt_off) = o[e];
-        }
-      }
+      for (int e = 0; e < 4; ++e) { qf[ks][e] = (int)lo[e]; qf[ks][4 + e] = (int)hi[e]; }
     }
+    // pin the loads here: the copies below are invisible to the compiler's wait counting
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) asm volatile("" : "+v"(qf[ks]));
+  }
+
+  // ---- global -> LDS copies: wavefront w copies rows 16w .. 16w+15 of every K and V tile with two
+  // instructions of 1 KB; lane l of instruction u lands at row 16w + 8u + l/8, chunk position l%8, and
+  // fetches the chunk that lives there.  Rows past the end of the chunk arrive as zeros. ---------------------
+  const u32x4 krs = rsrc_words(p.k + b * p.k_sb + hk * p.k_sh, (uint32_t)((int64_t)(p.Sc - 1) * p.k_ss + kD));
+  const u32x4 vrs = rsrc_words(p.v + b * p.v_sb + hk * p.v_sh, (uint32_t)((int64_t)(p.Sc - 1) * p.v_ss + kD));
+  int kvoff[2], vvoff[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int row = 16 * wave + 8 * u + (lane >> 3);
+    const int chunk = (lane & 7) ^ swz8(row);
+    kvoff[u] = (int)(row * p.k_ss) + chunk * 16;
+    vvoff[u] = (int)(row * p.v_ss) + chunk * 16;
+  }
+  const int k_tile_bytes = (int)(kBN * p.k_ss);
+  const int v_tile_bytes = (int)(kBN * p.v_ss);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem + wave * 2048;
+  auto copy_tile = [&](int t, int stage) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) copy16_to_lds(krs, lds_base + stage * kTileBytes + u * 1024, kvoff[u], t * k_tile_bytes);
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+      copy16_to_lds(vrs, lds_base + kVBase + stage * kTileBytes + u * 1024, vvoff[u], t * v_tile_bytes);
   };
 
-  const int k_rd = ln * kStride + hf * 16;            // + mb*32*144 + i*32
-  int v_rd[4];                                         // + (2 mb) * 16
+  // K operand of S^T: MFMA row m of block mb is key 32 mb + pi(m), pi(8 g + 4 h + e) = 16 h + 4 g + e, so
+  // that accumulator register i of lane half hf is key 32 mb + 16 hf + i.  The lane reads chunks
+  // 4 ks + 2 hf and 4 ks + 2 hf + 1 of that row.
+  const int pi = 16 * ((ln >> 2) & 1) + 4 * (ln >> 3) + (ln & 3);
+  int k_rd[2][2];                                     // [ks][second 16 bytes]  + mb * 4096
 #pragma unroll
-  for (int db = 0; db < 4; ++db) {
-    const int x = (db * 2 + (ln >> 4)) & 7;            // (d >> 4) & 7 for d = 32 db + ln
-    v_rd[db] = (db * 32 + (ln ^ x)) * kStride + hf * 16;
+  for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+    for (int u = 0; u < 2; ++u) k_rd[ks][u] = pi * 128 + (((4 * ks + 2 * hf + u) ^ swz8(pi)) << 4);
+  // V^T operand of O^T for head-dim block db and k-step ks2 (keys 64 ks2 .. +63): bytes 8 n .. 8 n + 7 of
+  // the lane's 32 are keys 64 ks2 + 32 (n / 2) + 16 hf + 8 (n % 2) + 0..7, the keys of its P registers.
+  // One ds_read_b64_tr_b8 per n: within 16 lanes, lane s supplies the address of row (first key) + s/2,
+  // head-dim bytes 8 (s%2) .. +7 of the 16-column strip, and receives column s.
+  int v_rd[4][2];                                     // [db][n % 2]  + ks2 * 8192 + (n / 2) * 4096
+  {
+    const int s16 = lane & 15, strip = (lane >> 4) & 1;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int o = 0; o < 2; ++o) {
+        const int row = 16 * hf + 8 * o + (s16 >> 1);
+        v_rd[db][o] = row * 128 + (((2 * db + strip) ^ swz8(row)) << 4) + (s16 & 1) * 8;
+      }
   }
+  typedef __attribute__((address_space(3))) i32x2* lds_i32x2;
+  auto read_k = [&](const unsigned char* ks_, int mb, int ks) -> i32x8 {
+    const u32x4 lo = *reinterpret_cast<const u32x4*>(ks_ + k_rd[ks][0] + mb * 4096);
+    const u32x4 hi = *reinterpret_cast<const u32x4*>(ks_ + k_rd[ks][1] + mb * 4096);
+    i32x8 r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { r[e] = (int)lo[e]; r[4 + e] = (int)hi[e]; }
+    return r;
+  };
+  auto read_v = [&](const unsigned char* vs_, int db, int ks2) -> i32x8 {
+    i32x8 r;
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      const i32x2 t = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+          (lds_i32x2)(vs_ + v_rd[db][n & 1] + ks2 * 8192 + (n >> 1) * 4096));
+      r[2 * n] = t[0]; r[2 * n + 1] = t[1];
+    }
+    return r;
+  };
   const int causal_shift = p.Sc - p.Sq;
 
   f32x16 o_acc[4];
@@ -172,28 +189,30 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
   float m_ref = -INFINITY, l_run = 0.f;      // l_run sums 2^7 P (this lane's half of the keys)
   const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
+  // Tile t lives in stage t % 4 of the K and the V ring.  An iteration starts by waiting for this
+  // wavefront's copies of tile t (those of tiles t+1 and t+2 stay in flight) and a barrier: after it tile t
+  // is complete for every wavefront and nobody reads tile t-1 any more, whose stages then receive tile t+3.
+  // Tiles past the end are copied as zeros so that the number of copies in flight stays the same.
   if (ntiles > 0) {
-    load_tile(0);
-    store_tile(0);
+    copy_tile(0, 0);
+    copy_tile(1, 1);
+    copy_tile(2, 2);
   }
   for (int t = 0; t < ntiles; ++t) {
-    const int stage = t & 1;
-    if (t + 1 < ntiles) load_tile(t + 1);
-    __syncthreads();
-    const unsigned char* ks = smem + stage * kStageBytes;
-    const unsigned char* vs = ks + kTileBytes;
+    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");      // two tiles of four copies each
+    __builtin_amdgcn_s_barrier();
+    copy_tile(t + 3, (t + 3) & 3);
+    const unsigned char* ks_ = smem + (t & 3) * kTileBytes;
+    const unsigned char* vs_ = smem + kVBase + (t & 3) * kTileBytes;
 
     // ---- S^T tile: 128 keys x 32 q rows per wave ------------------------------------------------------
     f32x16 s[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
       for (int mb = 0; mb < 4; ++mb) {
-        const u32x4 kf = *reinterpret_cast<const u32x4*>(ks + k_rd + mb * (32 * kStride) + i * 32);
-        s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(as_long(kf[0], kf[1]), as_long(qf[i][0], qf[i][1]),
-                                                           i == 0 ? zero : s[mb], 0, 0, 0);
-        s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(as_long(kf[2], kf[3]), as_long(qf[i][2], qf[i][3]),
-                                                           s[mb], 0, 0, 0);
+        const i32x8 kf = read_k(ks_, mb, ks);
+        s[mb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf[ks], ks == 0 ? zero : s[mb], 0, 0, 0, 0, 0, 0);
       }
     }
 
@@ -207,7 +226,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
       for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
-          const int key = kv0 + mb * 32 + (j >> 2) * 8 + hf * 4 + (j & 3);
+          const int key = kv0 + mb * 32 + hf * 16 + j;
           if (key > lim) s[mb][j] = -INFINITY;
         }
     }
@@ -232,7 +251,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
     }
     const float msc = (m_ref == -INFINITY) ? 0.f : m_ref * p.scale_log2 - kPShift;   // exponent of 2^7 P
     float rs = 0.f;
-    u32x4 pf[4];               // pf[mb]: dwords 0,1 = k-step (mb, 0), dwords 2,3 = k-step (mb, 1)
+    i32x8 pf[2];               // pf[ks2]: dwords 0-3 = keys of block 2 ks2, dwords 4-7 = block 2 ks2 + 1
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) {
 #pragma unroll
@@ -246,26 +265,22 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
         int packed = 0;
         packed = __builtin_amdgcn_cvt_pk_fp8_f32(s[mb][4 * w], s[mb][4 * w + 1], packed, false);
         packed = __builtin_amdgcn_cvt_pk_fp8_f32(s[mb][4 * w + 2], s[mb][4 * w + 3], packed, true);
-        pf[mb][w] = (uint32_t)packed;
+        pf[mb >> 1][(mb & 1) * 4 + w] = packed;
       }
     }
     l_run += rs;
 
     // ---- O^T += V^T P^T -----------------------------------------------------------------------------------
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb) {
+    for (int ks2 = 0; ks2 < 2; ++ks2) {
 #pragma unroll
       for (int db = 0; db < 4; ++db) {
-        const u32x4 vf = *reinterpret_cast<const u32x4*>(vs + v_rd[db] + mb * 32);
-        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(as_long(vf[0], vf[1]), as_long(pf[mb][0], pf[mb][1]),
-                                                               o_acc[db], 0, 0, 0);
-        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(as_long(vf[2], vf[3]), as_long(pf[mb][2], pf[mb][3]),
-                                                               o_acc[db], 0, 0, 0);
+        const i32x8 vf = read_v(vs_, db, ks2);
+        o_acc[db] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf[ks2], o_acc[db], 0, 0, 0, 0, 0, 0);
       }
     }
-
-    if (t + 1 < ntiles) store_tile(stage ^ 1);
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the zero-filled copies of tiles past the end
 
   // ---- epilogue ---------------------------------------------------------------------------------------------
   const float l_tot = pair_sum(l_run);
