@@ -44,6 +44,10 @@ BWD_SHAPES = [
     (1, 256, 256, 2, 2, True),
     (1, 200, 330, 2, 1, True),       # causal, bottom-right aligned, ragged
     (1, 330, 200, 2, 2, True),       # causal with rows that see no key
+    (1, 640, 640, 2, 1, True),       # causal GQA, ten streamed tiles per head: the LDS ring wraps twice
+    (1, 64, 700, 1, 1, False),       # few rows, many keys
+    (1, 700, 64, 3, 1, False),       # many rows of three grouped heads, few keys
+    (1, 1, 2, 1, 1, False),          # a single query row (with one key every gradient of q is exactly zero)
 ]
 
 

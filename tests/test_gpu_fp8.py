@@ -46,6 +46,7 @@ def _check(out, lse, ref_a, ref_b, tag, check_b=True):
 @pytest.mark.parametrize("B,Sq,Sc,Hq,Hkv,causal", [
     (1, 128, 128, 1, 1, False), (1, 256, 384, 2, 2, False), (2, 100, 77, 2, 1, False), (1, 300, 1000, 4, 2, False),
     (1, 256, 256, 2, 2, True), (1, 200, 330, 2, 1, True), (1, 130, 0, 1, 1, False),
+    (1, 520, 900, 2, 2, True), (1, 64, 1300, 1, 1, False), (1, 1, 1, 1, 1, False),
 ])
 def test_fp8_block_matches_oracle(B, Sq, Sc, Hq, Hkv, causal):
     import mercury_artifact_amd as M

@@ -55,6 +55,9 @@ SHAPES = [
     (1, 128, 320, 2, 2, True),      # causal with more keys than rows (bottom-right aligned)
     (1, 320, 128, 2, 2, True),      # causal with fewer keys: the first 192 rows see nothing
     (2, 130, 0, 2, 2, False),       # empty chunk
+    (1, 384, 1100, 2, 1, False),    # 18 tiles, ragged: the four-stage LDS ring wraps several times
+    (1, 384, 1100, 2, 1, True),
+    (1, 257, 63, 1, 1, False),      # one ragged tile, a second workgroup with a single row
 ]
 
 
