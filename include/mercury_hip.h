@@ -116,6 +116,15 @@ int mhip_lse_merge(const float* acc_out, const float* acc_lse,
 int mhip_flash_reduce(const float* lhs, const float* rhs, float* dst,
                       int64_t rows, int D, void* stream);
 
+/* Tree-attention merge of packed (rows, D+1) fp32 operands (out | lse) across ranks: replaces the local
+ * arithmetic of update_out_and_lse_collective, utils/flash_attn_dsl.py:307-324 (the collectives stay with
+ * the caller).  With row_max[r] = max over ranks of the lse column (one MAX all-reduce of `rows` floats):
+ *   finish == 0:  dst = (out * d | d), d = exp(lse - row_max)   -- this rank's term of ONE SUM all-reduce
+ *   finish != 0:  src is the summed terms; dst = (sum_out / sum_d | row_max + log(sum_d))
+ * dst may alias src.  Rows with row_max = -inf come out as (0 | -inf). */
+int mhip_tree_merge(const float* src, const float* row_max, float* dst, int64_t rows, int D, int finish,
+                    void* stream);
+
 /*
  * Pack a block result: dst (B,Sq,Hq,D+1) fp32 contiguous =
  * cat([float(block_out), block_lse^T], -1)   (utils/flash_attn_dsl.py:396).

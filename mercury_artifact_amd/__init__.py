@@ -11,13 +11,15 @@ from . import _native
 from .flash_attn_interface import (_flash_attn_backward, _flash_attn_forward, attn_bwd_block,
                                    attn_fwd_block)
 from .graph import GraphedStep
-from .merge import (_update_out_and_lse, flash_reduce, get_default_args, grad_accumulate, merge_into,
-                    pack_block, update_out_and_lse)
-from .ring import (flash_attn_backward, flash_attn_expose_reduce, flash_attn_pack_kv,
+from .merge import (LocalGroup, _update_out_and_lse, add_collective, flash_reduce, get_default_args,
+                    grad_accumulate, merge_into, pack_block, update_out_and_lse,
+                    update_out_and_lse_collective)
+from .ring import (flash_attn_backward, flash_attn_expose_reduce, flash_attn_expose_reduce_q_ring,
+                   flash_attn_pack_kv,
                    flash_attn_pack_split_kv, fp8_pack_split_kv, gqa_pack_kv, quantize_e4m3,
                    zigzag_causal_pack_kv)
 from .schedule import (LocalRing, double_ring_order, get_src_dst_ranks, n_dim_to_one_dim,
-                       one_dim_to_n_dim, ring_divide_order, shift_tuple_element, single_ring_order,
+                       one_dim_to_n_dim, reduce_buffer_route, ring_divide_order, shift_tuple_element, single_ring_order,
                        zigzag_blocks, zigzag_step)
 
 __version__ = "0.1.0"
@@ -33,6 +35,8 @@ def namespace() -> dict:
         "update_out_and_lse": update_out_and_lse,
         "_update_out_and_lse": _update_out_and_lse,
         "flash_reduce": flash_reduce,
+        "update_out_and_lse_collective": update_out_and_lse_collective,
+        "add_collective": add_collective,
         "one_dim_to_n_dim": one_dim_to_n_dim,
         "n_dim_to_one_dim": n_dim_to_one_dim,
         "shift_tuple_element": shift_tuple_element,

@@ -217,6 +217,62 @@ __global__ __launch_bounds__(256) void flash_reduce_kernel(const float* __restri
   }
 }
 
+// Tree-attention merge of packed (rows x W) = (out | lse) operands across ranks
+// (utils/flash_attn_dsl.py:307-324): with m = max over ranks of lse,
+//   prepare: dst = (out * d | d),  d = exp(lse - m)      -- what every rank contributes to the SUM
+//   finish:  dst = (sum_out / sum_d | m + log(sum_d))    -- from the summed contributions
+// Packing d next to out * d makes the SUM one collective instead of the reference's two.  Rows whose
+// lse is -inf everywhere (m = -inf) contribute d = 0 and finish as (0 | -inf).  Same flat walk in aligned
+// groups of four floats as flash_reduce_kernel; `aux` is the per-row maximum, contiguous.
+template <bool FINISH>
+__global__ __launch_bounds__(256) void tree_merge_kernel(const float* __restrict__ src,
+                                                         const float* __restrict__ aux,
+                                                         float* __restrict__ dst, int64_t total, int W) {
+  const int64_t g = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (g >= total) return;
+  float a[4];
+  if (g + 4 <= total) {
+    const f32x4 va = *reinterpret_cast<const f32x4*>(src + g);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) a[j] = va[j];
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) a[j] = g + j < total ? src[g + j] : 0.f;
+  }
+  const int64_t row_a = g / W;
+  const int64_t row_b = (g + 3) / W;
+  // per-row factor and last-column value, for the (at most) two rows this group touches
+  float f[2] = {0.f, 0.f}, last[2] = {0.f, 0.f};
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const int64_t row = k == 0 ? row_a : row_b;
+    if (k == 1 && (row_b == row_a || row_b * W + W - 1 >= total)) break;
+    const float m = aux[row];
+    const float tail = src[row * W + W - 1];
+    if (!FINISH) {
+      const float d = (m == -INFINITY) ? 0.f : __expf(tail - m);      // tail = this rank's lse
+      f[k] = d;
+      last[k] = d;
+    } else {
+      f[k] = tail > 0.f ? 1.f / tail : 0.f;                           // tail = summed d
+      last[k] = tail > 0.f ? m + __logf(tail) : -INFINITY;
+    }
+  }
+  float r[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int64_t e = g + j;
+    const int k = (e / W != row_a) ? 1 : 0;
+    r[j] = (e % W == W - 1) ? last[k] : a[j] * f[k];
+  }
+  if (g + 4 <= total) {
+    f32x4 v = {r[0], r[1], r[2], r[3]};
+    *reinterpret_cast<f32x4*>(dst + g) = v;
+  } else {
+    for (int j = 0; j < 4 && g + j < total; ++j) dst[g + j] = r[j];
+  }
+}
+
 // dst (rows x (D+1)) = pack(block)  or  flash_reduce(lhs, pack(block)); same flat walk over dst.
 template <bool REDUCE>
 __global__ __launch_bounds__(256) void pack_reduce_kernel(const float* __restrict__ lhs,
@@ -354,6 +410,21 @@ extern "C" int mhip_flash_reduce(const float* lhs, const float* rhs, float* dst,
   const int64_t groups = (total + 3) / 4;
   hipLaunchKernelGGL(flash_reduce_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), lhs, rhs, dst, total, D + 1);
+  return launch_status();
+}
+
+extern "C" int mhip_tree_merge(const float* src, const float* row_max, float* dst, int64_t rows, int D,
+                               int finish, void* stream) {
+  if (rows < 0 || D <= 0) return MHIP_EINVAL;
+  if (rows == 0) return MHIP_OK;
+  if (!src || !row_max || !dst) return MHIP_EINVAL;
+  if (!aligned16(src) || !aligned16(dst)) return MHIP_EALIGN;
+  const int64_t total = rows * (D + 1);
+  const int64_t groups = (total + 3) / 4;
+  const dim3 grid((unsigned)((groups + 255) / 256)), block(256);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (finish) hipLaunchKernelGGL(tree_merge_kernel<true>, grid, block, 0, st, src, row_max, dst, total, D + 1);
+  else hipLaunchKernelGGL(tree_merge_kernel<false>, grid, block, 0, st, src, row_max, dst, total, D + 1);
   return launch_status();
 }
 

@@ -8,14 +8,15 @@ from __future__ import annotations
 
 import inspect
 from functools import cache
-from typing import Optional, Tuple
+from typing import Optional, Sequence, Tuple
 
 import torch
 
 from . import _native as N
 
 __all__ = ["get_default_args", "update_out_and_lse", "_update_out_and_lse", "flash_reduce",
-           "pack_block", "merge_into", "grad_accumulate"]
+           "pack_block", "merge_into", "grad_accumulate", "update_out_and_lse_collective", "add_collective",
+           "LocalGroup"]
 
 
 @cache
@@ -126,6 +127,75 @@ def flash_reduce(lhs: torch.Tensor, rhs: torch.Tensor) -> torch.Tensor:
         code = N.lib().mhip_flash_reduce(N.ptr(lhs), N.ptr(rhs), N.ptr(dst), rows, W - 1, N.stream_of(lhs))
     N.check(code, "mhip_flash_reduce")
     return dst
+
+
+class LocalGroup:
+    """Single-GPU stand-in for the process group of a collective: ``peers`` are the operands of all ranks
+    of the group as they are when the collective starts, ``rank`` the position of the calling rank."""
+
+    def __init__(self, peers: Sequence[torch.Tensor], rank: int = 0):
+        if not 0 <= rank < len(peers):
+            raise ValueError("rank outside the group")
+        self.peers = list(peers)
+        self.rank = rank
+
+    def size(self) -> int:
+        return len(self.peers)
+
+
+def _is_collective(op, name: str) -> bool:
+    return op == name or getattr(op, "__name__", None) == name
+
+
+def _tree_merge(src: torch.Tensor, row_max: torch.Tensor, dst: torch.Tensor, finish: bool) -> None:
+    W = src.shape[-1]
+    rows = src.numel() // W if W else 0
+    with torch.cuda.device(src.device):
+        code = N.lib().mhip_tree_merge(N.ptr(src), N.ptr(row_max), N.ptr(dst), rows, W - 1, int(finish),
+                                       N.stream_of(src))
+    N.check(code, "mhip_tree_merge")
+
+
+def update_out_and_lse_collective(tensor: torch.Tensor, op, group: LocalGroup, dst: Optional[int] = None) -> None:
+    """utils/flash_attn_dsl.py:307-324: merge the packed ``(out | lse)`` partial results of all ranks of
+    ``group`` the tree-attention way (MAX of the lse, SUM of ``out * d`` and ``d``) and write the merged
+    value into ``tensor`` in place.  ``op`` is ``dist.all_reduce`` or ``dist.reduce`` (the function or its
+    name); with ``reduce`` only rank ``dst`` receives the result.  The per-rank arithmetic runs in two
+    kernels (``mhip_tree_merge``); the collectives themselves are replayed over ``group.peers``: one MAX
+    over the lse columns and ONE SUM over the packed ``(out * d | d)`` terms."""
+    reduce_to_one = _is_collective(op, "reduce")
+    if not (reduce_to_one or _is_collective(op, "all_reduce")):
+        raise RuntimeError("Unsupported collective op")
+    peers = [p.contiguous() for p in group.peers]
+    N.require_cuda(tensor, *peers)
+    for p in peers:
+        if p.shape != tensor.shape or p.dtype != torch.float32:
+            raise RuntimeError("all ranks contribute float32 tensors of one shape")
+    row_max = peers[0][..., -1].contiguous()
+    for p in peers[1:]:
+        row_max = torch.maximum(row_max, p[..., -1])          # the MAX all-reduce
+    total = None
+    for p in peers:
+        term = torch.empty_like(p)
+        _tree_merge(p, row_max, term, finish=False)
+        total = term if total is None else total.add_(term)   # the SUM all-reduce
+    if reduce_to_one and dst is not None and dst != group.rank:
+        return
+    out = tensor if tensor.is_contiguous() else torch.empty_like(total)
+    _tree_merge(total, row_max, out, finish=True)
+    if out is not tensor:
+        tensor.copy_(out)
+
+
+def add_collective(tensor: torch.Tensor, op, group: LocalGroup, dst: Optional[int] = None) -> None:
+    """utils/attn_bwd_dsl.py:28-35 as it is meant (the reference assigns the sum to a local name): the SUM
+    all-reduce of the gradient partials of all ranks of ``group``, written into ``tensor`` in place."""
+    if not _is_collective(op, "all_reduce"):
+        raise ValueError("not support other op than all reduce")
+    total = None
+    for p in group.peers:
+        total = p.to(torch.float32, copy=True) if total is None else total.add_(p)
+    tensor.copy_(total)
 
 
 def pack_block(block_out: torch.Tensor, block_lse: torch.Tensor,

@@ -16,9 +16,11 @@ import torch
 
 from .flash_attn_interface import _flash_attn_backward, _flash_attn_forward
 from .merge import get_default_args, grad_accumulate, merge_into, pack_block, update_out_and_lse
-from .schedule import LocalRing, n_dim_to_one_dim, one_dim_to_n_dim, shift_tuple_element, zigzag_step
+from .schedule import (LocalRing, n_dim_to_one_dim, one_dim_to_n_dim, reduce_buffer_route, shift_tuple_element,
+                       zigzag_step)
 
 __all__ = ["flash_attn_pack_kv", "gqa_pack_kv", "flash_attn_pack_split_kv", "flash_attn_expose_reduce",
+           "flash_attn_expose_reduce_q_ring",
            "flash_attn_backward", "zigzag_causal_pack_kv", "fp8_pack_split_kv", "quantize_e4m3"]
 
 
@@ -153,6 +155,49 @@ def flash_attn_expose_reduce(q, kv, o, lse, softmax_scale, dropout_p=0, causal=F
         buf = pack_block(block_out, block_lse, reduce_into=buf)
     o[:, :, :, :] = buf[..., :-1].to(o.dtype)
     lse[:, :, :] = buf[..., -1].transpose(1, 2)
+
+
+def flash_attn_expose_reduce_q_ring(qs, kvs, os_, lses, softmax_scale, dropout_p=0, causal=False,
+                                    window_size=(-1, -1), alibi_slopes=None, deterministic=False, *,
+                                    mesh_shape=None):
+    """The managed-reduction template (utils/flash_attn_dsl.py:345-408) scheduled as a ring over the
+    *reduce buffer*: every rank keeps its KV shard, Q and the packed partial result ``(out | lse)``
+    travel (codegen.py:116-190).  A rank's step is: block forward of the Q that just arrived against
+    the local KV, ``buf = flash_reduce(arrived_partial, pack(block))`` (one fused kernel), send on;
+    after the last step the buffer makes the write-back hop of ``get_src_dst_ranks``
+    (mercury/backend/pytorch/utils.py:171-192) to the rank that owns its Q rows.
+
+    What arrives at a rank was computed by the other ranks, so this driver runs ALL ranks of the mesh
+    in lock step on the one GPU: ``qs[r]``, ``kvs[r]`` are rank r's shards, ``os_[r]`` / ``lses[r]``
+    receive its result.  One rank's share of the work is 1 / world of the launches."""
+    world = len(qs)
+    mesh_shape = tuple(mesh_shape) if mesh_shape is not None else (world,)
+    sends, home_of = reduce_buffer_route(mesh_shape)
+    if len(home_of) != world or not (len(kvs) == len(os_) == len(lses) == world):
+        raise ValueError("need one q, kv, o and lse per rank of the mesh")
+    q_cur = list(qs)
+    arrived = [None] * world
+    home = [None] * world
+    for step in range(world):
+        buf = []
+        for r in range(world):
+            kv = kvs[r]
+            outputs = _flash_attn_forward(**_fwd_params(q_cur[r], kv[0], kv[1], softmax_scale, dropout_p, causal,
+                                                        window_size, alibi_slopes))
+            assert len(outputs) == 4
+            block_out, block_lse, _, _ = outputs
+            buf.append(pack_block(block_out, block_lse, reduce_into=arrived[r]))
+        if step + 1 != world:
+            q_next, arrived = [None] * world, [None] * world
+            for r in range(world):
+                q_next[sends[step][r]], arrived[sends[step][r]] = q_cur[r], buf[r]
+            q_cur = q_next
+        else:
+            for r in range(world):
+                home[home_of[r]] = buf[r]
+    for r in range(world):
+        os_[r][:, :, :, :] = home[r][..., :-1].to(os_[r].dtype)
+        lses[r][:, :, :] = home[r][..., -1].transpose(1, 2)
 
 
 def zigzag_causal_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=True, window_size=(-1, -1),

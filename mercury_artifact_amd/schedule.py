@@ -62,6 +62,31 @@ def get_src_dst_ranks(indices: Tuple[int, ...], mesh_shape: Tuple[int, ...],
     return n_dim_to_one_dim(src, tuple(mesh_shape)), n_dim_to_one_dim(dst, tuple(mesh_shape))
 
 
+def reduce_buffer_route(mesh_shape: Sequence[int]) -> Tuple[List[List[int]], List[int]]:
+    """Route of a ringed reduce buffer over the mesh (codegen.py:116-190): ``sends[s][r]`` is the rank
+    that rank ``r`` sends its buffer to after step ``s`` (innermost mesh dimension first, a hop on the
+    next dimension when the inner ring wraps), ``home[r]`` the destination of the write-back hop that
+    rank ``r`` makes after the last step (``get_src_dst_ranks``)."""
+    mesh_shape = tuple(int(x) for x in mesh_shape)
+    world = 1
+    for m in mesh_shape:
+        world *= m
+    sends: List[List[int]] = []
+    idx = [0] * len(mesh_shape)
+    for _ in range(world - 1):
+        dim = next(d for d in range(len(mesh_shape)) if idx[d] + 1 != mesh_shape[d])
+        sends.append([n_dim_to_one_dim(shift_tuple_element(one_dim_to_n_dim(r, mesh_shape), dim, 1, mesh_shape[dim]),
+                                       mesh_shape) for r in range(world)])
+        for d in range(len(mesh_shape)):      # advance the odometer (dimension 0 fastest)
+            idx[d] += 1
+            if idx[d] < mesh_shape[d]:
+                break
+            idx[d] = 0
+    dims = list(range(len(mesh_shape)))
+    home = [get_src_dst_ranks(one_dim_to_n_dim(r, mesh_shape), mesh_shape, dims)[1] for r in range(world)]
+    return sends, home
+
+
 # ------------------------------------------------------------------------------------------------
 # chunk order seen by one rank
 # ------------------------------------------------------------------------------------------------

@@ -32,7 +32,7 @@ import torch
 
 __all__ = [
     "block_attention", "single_pass_attention", "merge_reference", "merge_closed_form",
-    "update_out_and_lse", "pack_block", "flash_reduce", "block_backward",
+    "update_out_and_lse", "pack_block", "flash_reduce", "tree_merge", "block_backward",
     "single_ring_order", "double_ring_order", "ring_divide_order",
     "zigzag_blocks", "zigzag_step", "zigzag_local_positions",
     "quantize_e4m3", "dequantize",
@@ -153,6 +153,26 @@ def flash_reduce(lhs, rhs):
 # --------------------------------------------------------------------------------------
 # block backward  (contract of _flash_attn_backward at utils/attn_bwd_dsl.py:83-115)
 # --------------------------------------------------------------------------------------
+def tree_merge(packed_per_rank: Sequence[torch.Tensor]) -> torch.Tensor:
+    """Tree-attention merge of the packed ``(out | lse)`` partial results of all ranks, as
+    utils/flash_attn_dsl.py:307-324 does it with collectives: ``m = MAX lse``, ``d = exp(lse - m)``,
+    ``out = SUM(out * d) / SUM(d)``, ``lse = m + log SUM(d)``.  Rows that are -inf on every rank give
+    (0 | -inf) here (the reference would produce NaN).  Pinned in the tests against folding the same
+    operands pairwise with the closed-form merge."""
+    outs = [p[..., :-1].double() for p in packed_per_rank]
+    lses = [p[..., -1:].double() for p in packed_per_rank]
+    m = lses[0]
+    for l in lses[1:]:
+        m = torch.maximum(m, l)
+    safe_m = torch.where(torch.isinf(m), torch.zeros_like(m), m)
+    ds = [torch.exp(l - safe_m) for l in lses]
+    sum_d = sum(ds)
+    sum_out = sum(o * d for o, d in zip(outs, ds))
+    out = torch.where(sum_d > 0, sum_out / sum_d.clamp_min(1e-300), torch.zeros_like(sum_out))
+    lse = torch.where(sum_d > 0, m + torch.log(sum_d.clamp_min(1e-300)), torch.full_like(m, -math.inf))
+    return torch.cat([out, lse], dim=-1).to(packed_per_rank[0].dtype)
+
+
 def block_backward(dout, q, k, v, out, lse, softmax_scale, causal=False, dtype=torch.float32):
     """Gradients of one (Q shard, KV chunk) block given the *final merged* ``out`` and
     ``lse`` (utils/attn_bwd_dsl.py:73-76 loads them unchanged for every chunk).

@@ -122,3 +122,58 @@ def test_grad_accumulate(n):
     blk = torch.randn(n, generator=g).bfloat16()
     assert torch.equal(M.grad_accumulate(None, blk.cuda()).cpu(), blk.float())
     assert torch.equal(M.grad_accumulate(acc.cuda(), blk.cuda()).cpu(), acc + blk.float())
+
+
+@pytest.mark.parametrize("op", ["all_reduce", "reduce"])
+def test_tree_merge_collective_matches_oracle(op):
+    """update_out_and_lse_collective over a group of four ranks (collectives replayed on the one GPU)
+    against the CPU tree merge; one rank is all -inf, one row is -inf on every rank."""
+    import math
+
+    import mercury_artifact_amd as M
+
+    torch.manual_seed(8)
+    B, Sq, H, D, W = 2, 37, 3, 128, 4
+    peers = []
+    for r in range(W):
+        out = torch.randn(B, Sq, H, D)
+        lse = torch.randn(B, Sq, H, 1) * 3
+        if r == 2:
+            out.zero_()
+            lse.fill_(-math.inf)
+        lse[0, 5, 1] = -math.inf
+        out[0, 5, 1] = 0
+        peers.append(torch.cat([out, lse], dim=-1))
+    ref = O.tree_merge(peers)
+    dev = [p.cuda() for p in peers]
+    mine = dev[1].clone()
+    if op == "all_reduce":
+        M.update_out_and_lse_collective(mine, torch.distributed.all_reduce, M.LocalGroup(dev, rank=1))
+    else:
+        M.update_out_and_lse_collective(mine, "reduce", M.LocalGroup(dev, rank=1), dst=1)
+        other = dev[0].clone()
+        M.update_out_and_lse_collective(other, "reduce", M.LocalGroup(dev, rank=0), dst=1)
+        assert torch.equal(other, dev[0])                 # not the destination: untouched
+    torch.cuda.synchronize()
+    got = mine.cpu()
+    assert torch.equal(torch.isinf(got[..., -1]), torch.isinf(ref[..., -1]))
+    fin = ~torch.isinf(ref[..., -1])
+    assert (got[..., :-1] - ref[..., :-1]).abs().max().item() <= 2e-6
+    assert (got[..., -1][fin] - ref[..., -1][fin]).abs().max().item() <= 2e-6
+    assert (got[0, 5, 1, :-1] == 0).all()
+    for p, d in zip(peers, dev):
+        assert torch.equal(d.cpu(), p)                    # the other ranks' operands are not modified
+    with pytest.raises(RuntimeError):
+        M.update_out_and_lse_collective(mine, "reduce_scatter", M.LocalGroup(dev, rank=1))
+
+
+def test_add_collective_sums_the_group():
+    import mercury_artifact_amd as M
+
+    torch.manual_seed(9)
+    peers = [torch.randn(2, 16, 4, 128).cuda() for _ in range(3)]
+    mine = peers[0].clone()
+    M.add_collective(mine, "all_reduce", M.LocalGroup(peers, rank=0))
+    assert torch.allclose(mine, peers[0] + peers[1] + peers[2], atol=1e-6)
+    with pytest.raises(ValueError):
+        M.add_collective(mine, "reduce", M.LocalGroup(peers, rank=0))

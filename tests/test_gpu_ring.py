@@ -133,3 +133,27 @@ def test_zigzag_causal_ring(rank):
     lse = torch.empty(B, Hq, 2 * block, dtype=torch.float32, device="cuda")
     M.zigzag_causal_pack_kv(qd, dev[rank], o, lse, scale, ring=M.LocalRing((W,), rank, dev))
     _compare(o, lse, ref_o[:, pos[rank]], ref_l[:, :, pos[rank]])
+
+
+@pytest.mark.parametrize("mesh", [(4,), (4, 2)])
+def test_reduce_buffer_ring_all_ranks(mesh):
+    """Managed reduction scheduled as a ring over the packed partial result: Q and (out | lse) travel, KV
+    stays; after the write-back hop every rank must hold attention of its own Q rows over ALL keys."""
+    import mercury_artifact_amd as M
+
+    W = 1
+    for m in mesh:
+        W *= m
+    B, S, H, D = 1, 128 * W, 2, 128
+    q, k, v, qs, kvs = _inputs(B, S, H, H, D, W, seed=6)
+    scale = D ** -0.5
+    ref_o, ref_l = O.single_pass_attention(q.float(), k.float(), v.float(), scale)
+    Sc = S // W
+    qd = [x.cuda() for x in qs]
+    kvd = [x.cuda() for x in kvs]
+    outs = [torch.empty(B, Sc, H, D, dtype=torch.bfloat16, device="cuda") for _ in range(W)]
+    lses = [torch.empty(B, H, Sc, dtype=torch.float32, device="cuda") for _ in range(W)]
+    M.flash_attn_expose_reduce_q_ring(qd, kvd, outs, lses, scale, mesh_shape=mesh)
+    torch.cuda.synchronize()
+    for r in range(W):
+        _compare(outs[r], lses[r], ref_o[:, r * Sc:(r + 1) * Sc], ref_l[:, :, r * Sc:(r + 1) * Sc])

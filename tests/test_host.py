@@ -142,3 +142,23 @@ def test_quantize_e4m3_matches_oracle():
     a, sa = M.quantize_e4m3(x)
     b, sb = O.quantize_e4m3(x)
     assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)) and sa == sb
+
+
+@pytest.mark.parametrize("mesh", [(4,), (8,), (4, 2), (2, 3), (2, 2, 2)])
+def test_reduce_buffer_route_visits_every_rank_once_and_returns_home(mesh):
+    """Follow every ringed reduce buffer by hand: it must be at a different rank at every step (so it
+    folds in every KV shard exactly once) and the write-back hop must land it on the rank it started on."""
+    import mercury_artifact_amd as M
+
+    sends, home = M.reduce_buffer_route(mesh)
+    world = len(home)
+    assert len(sends) == world - 1
+    for start in range(world):
+        at, seen = start, [start]
+        for s in range(world - 1):
+            at = sends[s][at]
+            seen.append(at)
+        assert sorted(seen) == list(range(world))
+        assert home[at] == start
+    for s in range(world - 1):
+        assert sorted(sends[s]) == list(range(world))        # a hop is a permutation of the ranks

@@ -302,3 +302,32 @@ def test_quantize_e4m3_is_nearest_representable():
     assert ((got - y).abs() <= (nearest - y).abs() + 1e-7).all()
     assert got.abs().max() == 448.0
     assert torch.allclose(O.dequantize(xq, s), x, rtol=2 ** -4, atol=float(s) * 2 ** -9)
+
+
+def test_tree_merge_equals_pairwise_fold_and_single_pass():
+    """The tree-attention form (max, exp, sum, divide) is pinned by two things it must equal: folding the
+    same packed partials pairwise with the closed-form merge, and single-pass attention over all keys."""
+    torch.manual_seed(5)
+    B, Sq, H, D, W = 1, 24, 2, 16, 5
+    q = torch.randn(B, Sq, H, D, dtype=torch.float64)
+    k = torch.randn(B, W * 8, H, D, dtype=torch.float64)
+    v = torch.randn(B, W * 8, H, D, dtype=torch.float64)
+    parts = []
+    for c in range(W):
+        o, l = O.block_attention(q, k[:, c * 8:(c + 1) * 8], v[:, c * 8:(c + 1) * 8], 0.3, dtype=torch.float64)
+        parts.append(torch.cat([o, l.transpose(1, 2).unsqueeze(-1)], dim=-1))
+    tree = O.tree_merge(parts)
+    fold = parts[0]
+    for p in parts[1:]:
+        fold = O.flash_reduce(fold, p)
+    assert torch.allclose(tree, fold, atol=1e-12, rtol=1e-12)
+    ro, rl = O.single_pass_attention(q, k, v, 0.3, dtype=torch.float64)
+    assert torch.allclose(tree[..., :-1], ro, atol=1e-12)
+    assert torch.allclose(tree[..., -1], rl.transpose(1, 2), atol=1e-12)
+    # a rank that saw no key (lse = -inf) contributes nothing; all ranks empty -> (0 | -inf)
+    empty = torch.cat([torch.zeros(B, Sq, H, D, dtype=torch.float64),
+                       torch.full((B, Sq, H, 1), -math.inf, dtype=torch.float64)], dim=-1)
+    assert torch.allclose(O.tree_merge(parts + [empty]), tree, atol=1e-12)
+    both = O.tree_merge([empty, empty])
+    assert torch.equal(both[..., :-1], torch.zeros(B, Sq, H, D, dtype=torch.float64))
+    assert torch.isinf(both[..., -1]).all()
