@@ -90,6 +90,23 @@ def other_kernels(torch, M, dev):
                 n=5, w=2)
     out["fwd_e4m3_16384x16384"] = {"ms": round(ms, 4), "tflops": round(4.0 * B * H * S8 * S8 * D / ms / 1e9, 1),
                                    "pct_of_fp8_mfma_peak": round(4.0 * B * H * S8 * S8 * D / ms / 1e9 / 50.0, 2)}
+    # one rank's fp8 step over a 2 x 4 double ring: 8 chunks of 16384 keys, merges included
+    chunks8 = [torch.stack([k8, v8]) for _ in range(8)]          # timing only: every rank's chunk has the same bytes
+    ms = timeit(lambda: M.fp8_pack_split_kv(q8, chunks8[5], o8, l8, scale, sq, sk, sv,
+                                            ring=M.LocalRing((4, 2), 5, chunks8)), n=3, w=1)
+    out["step_e4m3_double_ring_16384x8"] = {"ms": round(ms, 3), "tflops": round(8 * 4.0 * B * H * S8 * S8 * D / ms / 1e9, 1)}
+    del q8, k8, v8, o8, l8, chunks8
+    # one rank's causal GQA step in the zigzag layout: B2, 32 q / 8 kv heads, 2 x 4096 local rows, 8 chunks
+    Bz, Hq, Hkv, Sz, W = 2, 32, 8, 8192, 8
+    qz = torch.randn(Bz, Sz, Hq, D, device=dev).bfloat16()
+    chunks = [torch.randn(2, Bz, Sz, Hkv, D, device=dev).bfloat16() for _ in range(W)]
+    oz = torch.empty_like(qz)
+    lz = torch.empty(Bz, Hq, Sz, dtype=torch.float32, device=dev)
+    ms = timeit(lambda: M.zigzag_causal_pack_kv(qz, chunks[0], oz, lz, scale, ring=M.LocalRing((W,), 0, chunks)),
+                n=5, w=2)
+    # a diagonal step and each of the 7 other steps cover half of a full 8192 x 8192 block
+    flops = (0.5 + 7 * 0.5) * 4.0 * Bz * Hq * Sz * Sz * D
+    out["step_bf16_zigzag_causal_gqa_8192x8"] = {"ms": round(ms, 3), "tflops": round(flops / ms / 1e9, 1)}
     return out
 
 
