@@ -120,35 +120,11 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
   const int hf = lane >> 5;
   const int my_r = r0 + wave * 32 + ln;             // this lane's stationary row
 
-  // ---- stationary operands: B operands of T1 / T2, lane (ln, hf) holds row[16 ks + 8 hf .. +7] -------
+  // ---- stationary operands: B operands of T1 / T2, lane (ln, hf) holds row[16 ks + 8 hf .. +7]; for dQ the
+  // query is the stationary row and its lse2 / delta are per-lane scalars.  All loaded further down, behind
+  // the first tile copies, so that one wait covers both latencies. ---------------------------------------
   bf16x8 xf[8], yf[8];
-  {
-    const int row = my_r < n_st ? my_r : n_st - 1;
-    const uint16_t* xp; const uint16_t* yp;
-    if (DQ) {
-      const int64_t off = b * p.q_sb + (int64_t)row * p.q_ss + hs * p.q_sh + hf * 8;
-      xp = p.q + off; yp = p.dout + off;
-    } else {
-      const int64_t off = b * p.k_sb + (int64_t)row * p.k_ss + hs * p.k_sh + hf * 8;
-      xp = p.k + off; yp = p.v + off;
-    }
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      xf[ks] = *reinterpret_cast<const bf16x8*>(xp + ks * 16);
-      yf[ks] = *reinterpret_cast<const bf16x8*>(yp + ks * 16);
-    }
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) { asm volatile("" : "+a"(xf[ks])); asm volatile("" : "+a"(yf[ks])); }
-  }
-  // DQ: the query is the stationary row, its lse2 / delta are per-lane scalars
   float lse2_lane = 0.f, delta_lane = 0.f;
-  if (DQ) {
-    const int row = my_r < n_st ? my_r : n_st - 1;
-    lse2_lane = p.lse2[((int64_t)b * p.Hq + hs) * p.Sq + row];
-    delta_lane = p.delta[((int64_t)b * p.Hq + hs) * p.Sq + row];
-  }
-  // pin the prologue loads here: the copies below are invisible to the compiler's wait counting
-  asm volatile("" : "+v"(lse2_lane), "+v"(delta_lane));
 
   // ---- streamed tiles ---------------------------------------------------------------------------------
   // DQ: K / V rows of kv head hs / group.  Otherwise: Q / dout rows of the `group` query heads that share
@@ -358,6 +334,32 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     copy_tile(0, 0);
     copy_tile(1, 1);
     copy_tile(2, 2);
+  }
+  {
+    const int row = my_r < n_st ? my_r : n_st - 1;
+    const uint16_t* xp; const uint16_t* yp;
+    if (DQ) {
+      const int64_t off = b * p.q_sb + (int64_t)row * p.q_ss + hs * p.q_sh + hf * 8;
+      xp = p.q + off; yp = p.dout + off;
+      lse2_lane = p.lse2[((int64_t)b * p.Hq + hs) * p.Sq + row];
+      delta_lane = p.delta[((int64_t)b * p.Hq + hs) * p.Sq + row];
+    } else {
+      const int64_t off = b * p.k_sb + (int64_t)row * p.k_ss + hs * p.k_sh + hf * 8;
+      xp = p.k + off; yp = p.v + off;
+    }
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      xf[ks] = *reinterpret_cast<const bf16x8*>(xp + ks * 16);
+      yf[ks] = *reinterpret_cast<const bf16x8*>(yp + ks * 16);
+    }
+    // Pin the loads here (the copies are invisible to the compiler's wait counting), the MFMA operands into
+    // accumulation registers: the arithmetic registers are needed for the tiles of T1 / T2 that the vector
+    // unit works on.
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) { asm volatile("" : "+a"(xf[ks])); asm volatile("" : "+a"(yf[ks])); }
+    asm volatile("" : "+v"(lse2_lane), "+v"(delta_lane));
+  }
+  if (ntiles > 0) {
     if (DQ) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
     static_assert(kCopiesPerTile == (DQ ? 8 : 9), "the vmcnt immediates are one and two tiles of copies");

@@ -103,17 +103,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
 
   // ---- Q fragment: B operand of S^T = K Q^T, lane (ln, hf) holds Q[row][16 ks + 8 hf .. +7] -----
   const int my_q = q0 + wave * 32 + ln;
-  bf16x8 qf[8];
-  {
-    const int row = my_q < p.Sq ? my_q : p.Sq - 1;
-    const uint16_t* qp = p.q + b * p.q_sb + (int64_t)row * p.q_ss + hq * p.q_sh + hf * 8;
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qp + ks * 16);
-    // Pin the fragment here: otherwise its first use sits inside the main loop and the wait for
-    // these loads lands there, where it also waits for the tile prefetch issued just before it.
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) asm volatile("" : "+v"(qf[ks]));
-  }
+  bf16x8 qf[8];   // loaded in the prologue, after the first tile copies are under way
 
   // ---- global -> LDS copies of the K and V tiles ---------------------------------------------------
   // A tile is 64 rows of 256 bytes.  Chunk c (16 bytes) of row r lives at chunk position c ^ swz(r):
@@ -353,6 +343,18 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     for (int i = 0; i < kStages; ++i) copy_k(i, i);          // tiles past the chunk arrive as zeros
 #pragma unroll
     for (int i = 0; i < kStages - 1; ++i) copy_v(i, i);
+  }
+  {
+    // The Q loads go out behind the copies, so that one wait covers both latencies.  The fragment is
+    // pinned here: otherwise its first use sits inside the main loop and so does the wait for it.
+    const int row = my_q < p.Sq ? my_q : p.Sq - 1;
+    const uint16_t* qp = p.q + b * p.q_sb + (int64_t)row * p.q_ss + hq * p.q_sh + hf * 8;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qp + ks * 16);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) asm volatile("" : "+v"(qf[ks]));
+  }
+  if (ntiles > 0) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     qk(0);

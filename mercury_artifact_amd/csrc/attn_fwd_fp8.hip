@@ -96,21 +96,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
 
   // ---- Q fragment: B operand of S^T, lane (ln, hf) holds bytes [64 ks + 32 hf, +32) of its row ------------
   const int my_q = q0 + wave * 32 + ln;
-  i32x8 qf[2];
-  {
-    const int row = my_q < p.Sq ? my_q : p.Sq - 1;
-    const uint8_t* qp = p.q + b * p.q_sb + (int64_t)row * p.q_ss + hq * p.q_sh + hf * 32;
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      const u32x4 lo = *reinterpret_cast<const u32x4*>(qp + ks * 64);
-      const u32x4 hi = *reinterpret_cast<const u32x4*>(qp + ks * 64 + 16);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) { qf[ks][e] = (int)lo[e]; qf[ks][4 + e] = (int)hi[e]; }
-    }
-    // pin the loads here: the copies below are invisible to the compiler's wait counting
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) asm volatile("" : "+v"(qf[ks]));
-  }
+  i32x8 qf[2];    // loaded after the first tile copies are under way, so that one wait covers both latencies
 
   // ---- global -> LDS copies: wavefront w copies rows 16w .. 16w+15 of every K and V tile with two
   // instructions of 1 KB; lane l of instruction u lands at row 16w + 8u + l/8, chunk position l%8, and
@@ -197,6 +183,20 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
     copy_tile(0, 0);
     copy_tile(1, 1);
     copy_tile(2, 2);
+  }
+  {
+    const int row = my_q < p.Sq ? my_q : p.Sq - 1;
+    const uint8_t* qp = p.q + b * p.q_sb + (int64_t)row * p.q_ss + hq * p.q_sh + hf * 32;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const u32x4 lo = *reinterpret_cast<const u32x4*>(qp + ks * 64);
+      const u32x4 hi = *reinterpret_cast<const u32x4*>(qp + ks * 64 + 16);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { qf[ks][e] = (int)lo[e]; qf[ks][4 + e] = (int)hi[e]; }
+    }
+    // pin the loads here: the copies are invisible to the compiler's wait counting
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) asm volatile("" : "+v"(qf[ks]));
   }
   for (int t = 0; t < ntiles; ++t) {
     asm volatile("s_waitcnt vmcnt(8)" ::: "memory");      // two tiles of four copies each
