@@ -68,3 +68,26 @@ def test_graphed_backward_block_matches_eager():
         graphed.replay()
         torch.cuda.synchronize()
         assert torch.equal(dq, edq) and torch.equal(dkv, edkv), it
+
+
+def test_search_harness_times_a_step():
+    """bench_callable follows the timing protocol of the reference's schedule search: warm-up, timed calls
+    between device events, (iterations per second, seconds, bytes)."""
+    import mercury_artifact_amd as M
+    from mercury_artifact_amd import search_harness as SH
+
+    B, S, H, D, W = 1, 256, 2, 128, 2
+    q = torch.randn(B, S, H, D, device="cuda").bfloat16()
+    chunks = [torch.randn(2, B, S, H, D, device="cuda").bfloat16() for _ in range(W)]
+    o = torch.zeros_like(q)
+    lse = torch.zeros(B, H, S, dtype=torch.float32, device="cuda")
+
+    def step(q, kv, o, lse):
+        M.flash_attn_pack_kv(q, kv, o, lse, D ** -0.5, ring=M.LocalRing((W,), 0, chunks))
+
+    ips, seconds, nbytes = SH.bench_callable(step, {"q": q, "kv": chunks[0], "o": o, "lse": lse}, num_iter=5)
+    assert ips > 0 and seconds > 0 and abs(ips * seconds - 5) < 1e-6
+    assert nbytes == sum(t.numel() * t.element_size() for t in (q, chunks[0], o, lse))
+    assert o.float().abs().max().item() > 0
+    with pytest.raises(ImportError):
+        SH.bench_program(object())          # the IR and its code generator are not part of this package
