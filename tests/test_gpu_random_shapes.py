@@ -1,0 +1,96 @@
+"""Seeded random small shapes through the three block kernels against the CPU oracle: ragged row and key
+counts, batch 1-3, 1-4 query heads per KV head, with and without the causal mask.  Tolerances as in the
+per-kernel test files."""
+import random
+
+import pytest
+import torch
+
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _shapes(seed, n, max_s):
+    rng = random.Random(seed)
+    out = []
+    for _ in range(n):
+        hkv = rng.randint(1, 2)
+        out.append((rng.randint(1, 3), rng.randint(1, max_s), rng.randint(1, max_s), hkv * rng.randint(1, 4), hkv,
+                    rng.random() < 0.5))
+    return out
+
+
+@pytest.mark.parametrize("B,Sq,Sc,Hq,Hkv,causal", _shapes(101, 16, 420))
+def test_random_forward(B, Sq, Sc, Hq, Hkv, causal):
+    import mercury_artifact_amd as M
+
+    print(f"fwd B{B} Sq{Sq} Sc{Sc} Hq{Hq} Hkv{Hkv} causal={causal}", flush=True)
+    g = torch.Generator().manual_seed(B * 1000003 + Sq * 1009 + Sc)
+    q = torch.randn(B, Sq, Hq, 128, generator=g).bfloat16()
+    kv = torch.randn(2, B, Sc, Hkv, 128, generator=g).bfloat16()
+    scale = 128 ** -0.5
+    ro, rl = O.block_attention(q.float(), kv[0].float(), kv[1].float(), scale, causal=causal)
+    out, lse = M.attn_fwd_block(q.cuda(), kv[0].cuda(), kv[1].cuda(), scale, causal=causal)
+    out, lse = out.float().cpu(), lse.cpu()
+    assert torch.equal(torch.isinf(lse), torch.isinf(rl))
+    assert (out - ro).abs().max().item() <= 2e-2
+    if ro.norm().item() > 0:
+        assert (out - ro).norm().item() / ro.norm().item() <= 1e-2
+    fin = ~torch.isinf(rl)
+    if fin.any():
+        assert ((lse[fin] - rl[fin]).abs() / rl[fin].abs().clamp_min(1.0)).max().item() <= 1e-3
+
+
+@pytest.mark.parametrize("B,Sq,Sc,Hq,Hkv,causal", _shapes(202, 12, 300))
+def test_random_backward(B, Sq, Sc, Hq, Hkv, causal):
+    import mercury_artifact_amd as M
+
+    print(f"bwd B{B} Sq{Sq} Sc{Sc} Hq{Hq} Hkv{Hkv} causal={causal}", flush=True)
+    g = torch.Generator().manual_seed(B * 1000003 + Sq * 1009 + Sc + 7)
+    q = torch.randn(B, Sq, Hq, 128, generator=g).bfloat16()
+    kv = torch.randn(2, B, Sc, Hkv, 128, generator=g).bfloat16()
+    dout = torch.randn(B, Sq, Hq, 128, generator=g).bfloat16()
+    scale = 128 ** -0.5
+    o, lse = O.block_attention(q.float(), kv[0].float(), kv[1].float(), scale, causal=causal)
+    o16 = o.bfloat16()
+    refs = O.block_backward(dout.float(), q.float(), kv[0].float(), kv[1].float(), o16.float(), lse, scale,
+                            causal=causal)
+    qd, kvd = q.cuda(), kv.cuda()
+    dq = torch.full_like(qd, float("nan"))
+    dkv = torch.full_like(kvd, float("nan"))
+    M.attn_bwd_block(dout.cuda(), qd, kvd[0], kvd[1], o16.cuda(), lse.cuda(), dq, dkv[0], dkv[1], scale, causal=causal)
+    for name, got, ref in (("dq", dq, refs[0]), ("dk", dkv[0], refs[1]), ("dv", dkv[1], refs[2])):
+        got = got.float().cpu()
+        assert not torch.isnan(got).any(), name
+        scale_ref = ref.abs().max().item()
+        assert (got - ref).abs().max().item() <= 4e-2 * scale_ref + 1e-6, name
+        if ref.norm().item() > 1e-3:
+            assert (got - ref).norm().item() / ref.norm().item() <= 1.5e-2, name
+
+
+@pytest.mark.parametrize("B,Sq,Sc,Hq,Hkv,causal", _shapes(303, 10, 500))
+def test_random_fp8_forward(B, Sq, Sc, Hq, Hkv, causal):
+    import mercury_artifact_amd as M
+
+    print(f"fp8 B{B} Sq{Sq} Sc{Sc} Hq{Hq} Hkv{Hkv} causal={causal}", flush=True)
+    g = torch.Generator().manual_seed(B * 1000003 + Sq * 1009 + Sc + 13)
+    q = torch.randn(B, Sq, Hq, 128, generator=g)
+    k = torch.randn(B, Sc, Hkv, 128, generator=g)
+    v = torch.randn(B, Sc, Hkv, 128, generator=g)
+    (qq, sq), (kq, sk), (vq, sv) = O.quantize_e4m3(q), O.quantize_e4m3(k), O.quantize_e4m3(v)
+    scale = 128 ** -0.5
+    oa, la = O.block_attention(O.dequantize(qq, sq), O.dequantize(kq, sk), O.dequantize(vq, sv), scale, causal=causal)
+    out, lse = M.attn_fwd_block(qq.cuda(), kq.cuda(), vq.cuda(), scale, causal=causal,
+                                q_descale=sq.cuda(), k_descale=sk.cuda(), v_descale=sv.cuda())
+    out, lse = out.float().cpu(), lse.cpu()
+    assert torch.equal(torch.isinf(lse), torch.isinf(la))
+    # own per-element bound against attention on the de-quantised inputs: 4e-2 + 2^-4 |ref| (rows that see two or
+    # three keys of opposite sign can cancel in |ref| but not in the rounding error of P), inside the stated
+    # fp8 bar of 6e-2
+    assert ((out - oa).abs() - (4e-2 + 2 ** -4 * oa.abs())).max().item() <= 0
+    if oa.norm().item() > 0:
+        assert (out - oa).norm().item() / oa.norm().item() <= 6e-2
+    fin = ~torch.isinf(la)
+    if fin.any():
+        assert ((lse[fin] - la[fin]).abs() / la[fin].abs().clamp_min(1.0)).max().item() <= 1e-3
