@@ -295,16 +295,26 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     l = *(lds_f32x4)(uintptr_t)(uint32_t)addr;
     d = *(lds_f32x4)(uintptr_t)(uint32_t)(addr + (kOffDelta - kOffLse));
   };
-  // P / dS of accumulator register i of the half in (c1, c2), packed into B operands every 8 registers
-  auto vector_slot = [&](int i, f32x16& c1, f32x16& c2, int stage, int mb) {
-    if (!DQ && (i & 3) == 0 && i < 12) read_ld(stage, mb, (i >> 2) + 1, lv[(i >> 2) + 1], dv[(i >> 2) + 1]);
-    const float l = DQ ? lse2_lane : lv[i >> 2][i & 3];
-    const float d = DQ ? delta_lane : dv[i >> 2][i & 3];
-    const float pe = fast_exp2(__builtin_fmaf(c1[i], p.scale_log2, -l));
-    c1[i] = pe;
-    c2[i] = pe * (c2[i] - d);
-    if ((i & 7) == 7) {
-      const int j2 = i >> 3;
+  // P / dS of the half in (c1, c2), one accumulator register per slot, as a three-stage pipeline so that
+  // no instruction waits for the one issued just before it (a wavefront issues in order):
+  //   slot s:  argument of the exponential and dP - delta of register s      (s < 16)
+  //            exponential of register s - 1                                 (1 <= s < 17)
+  //            dS = P (dP - delta) of register s - 2                         (2 <= s < 18)
+  // and the packing into B operands once 8 registers are through (slots 9 and 17).  Slots 16 and 17 ride on
+  // the first two slots of the accumulate phase that follows.
+  float earg[16];
+  auto vector_slot = [&](int s, f32x16& c1, f32x16& c2, int stage, int mb) {
+    if (s < 16) {
+      if (!DQ && (s & 3) == 0 && s < 12) read_ld(stage, mb, (s >> 2) + 1, lv[(s >> 2) + 1], dv[(s >> 2) + 1]);
+      const float l = DQ ? lse2_lane : lv[s >> 2][s & 3];
+      const float d = DQ ? delta_lane : dv[s >> 2][s & 3];
+      earg[s] = __builtin_fmaf(c1[s], p.scale_log2, -l);
+      c2[s] = c2[s] - d;
+    }
+    if (s >= 1 && s < 17) c1[s - 1] = fast_exp2(earg[s - 1]);
+    if (s >= 2 && s < 18) c2[s - 2] = c1[s - 2] * c2[s - 2];
+    if (s == 9 || s == 17) {
+      const int j2 = s >> 4;
       u32x4 wp, wd;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -396,6 +406,7 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     }
 #pragma unroll
     for (int i = 0; i < kAcc; ++i) {                     // P1
+      if (i < 2) vector_slot(16 + i, ta1, ta2, stage, 0);
       acc_mfma(i, ring[(kP1 + i) % kDepth]);
       if (!DQ && i == kAcc - 2) read_ld(stage, 1, 0, lv[0], dv[0]);
       ring[(kP1 + i) % kDepth] = read_slot(kP1 + i + kDepth);
@@ -411,6 +422,7 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     }
 #pragma unroll
     for (int i = 0; i < kAcc; ++i) {                     // P3
+      if (i < 2) vector_slot(16 + i, tb1, tb2, stage, 1);
       acc_mfma(i, ring[(kP3 + i) % kDepth]);
       if (!DQ && i == kAcc - 2) read_ld((t + 1) & 3, 0, 0, lv[0], dv[0]);
       ring[(kP3 + i) % kDepth] = read_slot(kP3 + i + kDepth);
