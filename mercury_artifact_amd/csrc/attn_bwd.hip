@@ -193,6 +193,26 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     }
   };
   constexpr int kCopiesPerTile = DQ ? 8 : 9;
+  // The same copies one instruction at a time (piece 0 .. kCopiesPerTile - 1), so that the main loop can
+  // issue them between MFMAs; the scalar offsets are worked out once per tile by copy_setup.
+  int cp_soff = 0, cp_hq = 0, cp_c0 = 0;
+  bool cp_live = false;
+  auto copy_setup = [&](int t) {
+    cp_live = t < ntiles;
+    cp_hq = DQ ? 0 : hs * p.group + tile_head(cp_live ? t : 0);
+    cp_c0 = tile_row0(cp_live ? t : 0);
+    cp_soff = cp_live ? (int)(((int64_t)cp_c0 * s_ss + (int64_t)cp_hq * s_sh) * 2) : kNoTile;
+  };
+  auto copy_piece = [&](int piece, int stage) {
+    const uint32_t dst = lds_base + stage * kStageBytes + wave * 4096;
+    if (piece < 4) copy16_to_lds(xrs, dst + piece * 1024, cvoff[piece], cp_soff);
+    else if (piece < 8) copy16_to_lds(yrs, dst + kOffY + (piece - 4) * 1024, cvoff[piece - 4], cp_soff);
+    else if (!DQ) {
+      const float* src = ((wave & 1) ? p.delta : p.lse2) + ((int64_t)b * p.Hq + cp_hq) * p.Sq;
+      copy4_to_lds(rsrc_words(src, (uint32_t)p.Sq * 4u), lds_base + stage * kStageBytes + ((wave & 1) ? kOffDelta : kOffLse),
+                   lane * 4, cp_live ? cp_c0 * 4 : kNoTile);
+    }
+  };
 
   // row-major operand reads (A of T1 / T2): lane (ln, hf) reads chunk 2 kk + hf of row 32 mb + ln
   int rm_rd[8];                                       // + mb * 8192
@@ -295,36 +315,50 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     l = *(lds_f32x4)(uintptr_t)(uint32_t)addr;
     d = *(lds_f32x4)(uintptr_t)(uint32_t)(addr + (kOffDelta - kOffLse));
   };
-  // P / dS of the half in (c1, c2), one accumulator register per slot, as a three-stage pipeline so that
-  // no instruction waits for the one issued just before it (a wavefront issues in order):
-  //   slot s:  argument of the exponential and dP - delta of register s      (s < 16)
-  //            exponential of register s - 1                                 (1 <= s < 17)
-  //            dS = P (dP - delta) of register s - 2                         (2 <= s < 18)
-  // and the packing into B operands once 8 registers are through (slots 9 and 17).  Slots 16 and 17 ride on
-  // the first two slots of the accumulate phase that follows.
+  // P / dS of the half in (c1, c2): 16 accumulator registers, spread over the 16 slots in which the next
+  // half's T1 / T2 are issued AND the first slots of the accumulate phase that follows (a wavefront issues
+  // one vector instruction every ~5 cycles, so 16 slots of 32 cycles do not hold all of it).  Register e
+  // enters at slot first_slot(e); its work is a three-stage pipeline so that no instruction waits for the
+  // one issued just before it:
+  //   first_slot      argument of the exponential, dP - delta
+  //   first_slot + 1  exponential
+  //   first_slot + 2  dS = P (dP - delta)
+  // Registers 0-7 (k-step 0 of the accumulate phase) are packed before that phase starts, registers 8-15
+  // before its second half does.
+  auto first_slot = [](int e) -> int {
+    if (DQ) return e < 8 ? (e * 3) / 2 : 1 + e;          // 0,1,3,4,6,7,9,10 | 9..16: packed at slots 13 and 19 (acc 16-19, 20-23)
+    return e < 8 ? (e * 7) / 4 : 5 + e;                  // 0,1,3,5,7,8,10,12 | 13..20: packed at slots 15 and 23 (acc 16-23, 24-31)
+  };
   float earg[16];
   auto vector_slot = [&](int s, f32x16& c1, f32x16& c2, int stage, int mb) {
-    if (s < 16) {
-      if (!DQ && (s & 3) == 0 && s < 12) read_ld(stage, mb, (s >> 2) + 1, lv[(s >> 2) + 1], dv[(s >> 2) + 1]);
-      const float l = DQ ? lse2_lane : lv[s >> 2][s & 3];
-      const float d = DQ ? delta_lane : dv[s >> 2][s & 3];
-      earg[s] = __builtin_fmaf(c1[s], p.scale_log2, -l);
-      c2[s] = c2[s] - d;
-    }
-    if (s >= 1 && s < 17) c1[s - 1] = fast_exp2(earg[s - 1]);
-    if (s >= 2 && s < 18) c2[s - 2] = c1[s - 2] * c2[s - 2];
-    if (s == 9 || s == 17) {
-      const int j2 = s >> 4;
-      u32x4 wp, wd;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        wp[e] = pack_bf16(c1[8 * j2 + 2 * e], c1[8 * j2 + 2 * e + 1]);
-        wd[e] = pack_bf16(c2[8 * j2 + 2 * e], c2[8 * j2 + 2 * e + 1]);
+    for (int e = 0; e < 16; ++e) {
+      const int f = first_slot(e);
+      if (s == f) {
+        const float l = DQ ? lse2_lane : lv[e >> 2][e & 3];
+        const float d = DQ ? delta_lane : dv[e >> 2][e & 3];
+        earg[e] = __builtin_fmaf(c1[e], p.scale_log2, -l);
+        c2[e] = c2[e] - d;
+        // lse2 / delta of the next four rows, one group ahead
+        if (!DQ && (e & 3) == 0 && e < 12) read_ld(stage, mb, (e >> 2) + 1, lv[(e >> 2) + 1], dv[(e >> 2) + 1]);
       }
-      pfrag[j2] = __builtin_bit_cast(bf16x8, wp);
-      dsfrag[j2] = __builtin_bit_cast(bf16x8, wd);
+      if (s == f + 1) c1[e] = fast_exp2(earg[e]);
+      if (s == f + 2) c2[e] = c1[e] * c2[e];
     }
+#pragma unroll
+    for (int j2 = 0; j2 < 2; ++j2)
+      if (s == first_slot(8 * j2 + 7) + 3) {
+        u32x4 wp, wd;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          wp[e] = pack_bf16(c1[8 * j2 + 2 * e], c1[8 * j2 + 2 * e + 1]);
+          wd[e] = pack_bf16(c2[8 * j2 + 2 * e], c2[8 * j2 + 2 * e + 1]);
+        }
+        pfrag[j2] = __builtin_bit_cast(bf16x8, wp);
+        dsfrag[j2] = __builtin_bit_cast(bf16x8, wd);
+      }
   };
+  constexpr int kVecTail = DQ ? 4 : 8;      // accumulate-phase slots that still carry vector work
   auto acc_mfma = [&](int i, const bf16x8& a) {
     const int m = DQ ? i : (i >> 1);
     const int db = m & 3, j2 = m >> 2;
@@ -393,20 +427,22 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     if (DQ) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
     __builtin_amdgcn_s_barrier();
-    copy_tile(t + 3, (t + 3) & 3);
-    tile_addrs((t + 1) & 3, rm_n, tr_n);
+    copy_setup(t + 3);
+    const int next_base = (int)lds_base + ((t + 1) & 3) * kStageBytes;
     static_assert(kSlots % kDepth == 0 && 16 % kDepth == 0, "the ring position is the slot number modulo its depth");
     mask_half(ta1, c0);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {                       // P0
+    for (int i = 0; i < 16; ++i) {                       // P0, carrying the copies of tile t+3
       t_mfma(i, ring[i % kDepth], tb1, tb2);
       vector_slot(i, ta1, ta2, stage, 0);
+      if (i < kCopiesPerTile) copy_piece(i, (t + 3) & 3);
+      if (i >= 8) rm_n[i - 8] = rm_rd[i - 8] + next_base;          // needed from P2 on (after slot kP2 - kDepth)
       ring[i % kDepth] = read_slot(i + kDepth);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int i = 0; i < kAcc; ++i) {                     // P1
-      if (i < 2) vector_slot(16 + i, ta1, ta2, stage, 0);
+      if (i < kVecTail) vector_slot(16 + i, ta1, ta2, stage, 0);
       acc_mfma(i, ring[(kP1 + i) % kDepth]);
       if (!DQ && i == kAcc - 2) read_ld(stage, 1, 0, lv[0], dv[0]);
       ring[(kP1 + i) % kDepth] = read_slot(kP1 + i + kDepth);
@@ -417,12 +453,13 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     for (int i = 0; i < 16; ++i) {                       // P2
       t_mfma(i, ring[(kP2 + i) % kDepth], ta1, ta2);
       vector_slot(i, tb1, tb2, stage, 1);
+      if (i < 8) { const int db = i >> 1, h = i & 1; tr_n[db][h] = tr_rd[db][h] + next_base; }   // for the next tile
       ring[(kP2 + i) % kDepth] = read_slot(kP2 + i + kDepth);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int i = 0; i < kAcc; ++i) {                     // P3
-      if (i < 2) vector_slot(16 + i, tb1, tb2, stage, 1);
+      if (i < kVecTail) vector_slot(16 + i, tb1, tb2, stage, 1);
       acc_mfma(i, ring[(kP3 + i) % kDepth]);
       if (!DQ && i == kAcc - 2) read_ld((t + 1) & 3, 0, 0, lv[0], dv[0]);
       ring[(kP3 + i) % kDepth] = read_slot(kP3 + i + kDepth);
