@@ -1,0 +1,83 @@
+"""Argument validation of the C ABI: every rejected call returns its error code before anything is launched,
+so these run without a GPU (the pointers are never dereferenced)."""
+import ctypes
+
+import pytest
+
+from mercury_artifact_amd import _native as N
+
+OK, EINVAL, EDTYPE, EHEADDIM, EALIGN, EUNSUPPORTED = 0, -1, -2, -3, -4, -6
+P = 0x10000           # a non-NULL, 16-byte aligned "pointer"
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return N.lib()
+
+
+def _fwd(lib, q=P, k=P, v=P, out=P, lse=P, B=1, Sq=64, Sc=64, Hq=2, Hkv=2, D=128,
+         strides=None, scale=0.1, mask=0, dtype=0, descales=(1.0, 1.0, 1.0)):
+    if strides is None:
+        strides = [Sq * Hq * D, Hq * D, D, Sc * Hkv * D, Hkv * D, D, Sc * Hkv * D, Hkv * D, D, Sq * Hq * D, Hq * D, D]
+    return lib.mhip_attn_fwd_block(q, k, v, out, lse, B, Sq, Sc, Hq, Hkv, D, *strides, scale, mask, dtype,
+                                   *descales, None)
+
+
+def test_forward_rejects(lib):
+    assert _fwd(lib, D=64) == EHEADDIM
+    assert _fwd(lib, Hq=3, Hkv=2) == EINVAL
+    assert _fwd(lib, Sq=-1) == EINVAL
+    assert _fwd(lib, scale=0.0) == EINVAL
+    assert _fwd(lib, scale=float("inf")) == EINVAL
+    assert _fwd(lib, scale=float("nan")) == EINVAL
+    assert _fwd(lib, mask=2) == EINVAL
+    assert _fwd(lib, dtype=7) == EDTYPE
+    assert _fwd(lib, q=None) == EINVAL
+    assert _fwd(lib, k=None) == EINVAL
+    assert _fwd(lib, q=P + 8) == EALIGN
+    s = [64 * 2 * 128, 2 * 128, 128] * 4
+    s[1] += 4                                   # a row stride that breaks 16-byte alignment
+    assert _fwd(lib, strides=s) == EALIGN
+    big = 1 << 20                               # rows 2 MiB apart: 2048 of them span 4 GiB
+    assert _fwd(lib, Sc=2048, strides=[64 * 256, 256, 128, 2048 * big, big, 128, 2048 * big, big, 128,
+                                       64 * 256, 256, 128]) == EUNSUPPORTED
+    assert _fwd(lib, dtype=1, descales=(1.0, 0.0, 1.0)) == EINVAL
+    # nothing to do: accepted without touching the pointers
+    assert _fwd(lib, B=0) == OK
+    assert _fwd(lib, Sq=0) == OK
+    assert lib.mhip_error_string(EHEADDIM).startswith(b"head dimension")
+
+
+def test_backward_rejects(lib):
+    def bwd(B=1, Sq=64, Sc=64, Hq=2, Hkv=2, D=128, scale=0.1, mask=0, dq=P, ws=P, strides=None, dq_acc=None):
+        if strides is None:
+            strides = [Sq * Hq * D, Hq * D, D, Sc * Hkv * D, Hkv * D, D, Sc * Hkv * D, Hkv * D, D]
+        return lib.mhip_attn_bwd_block(P, P, P, P, P, P, dq, P, P, dq_acc, B, Sq, Sc, Hq, Hkv, D, *strides,
+                                       scale, mask, 0, ws, None)
+
+    assert bwd(D=96) == EHEADDIM
+    assert bwd(Hq=5, Hkv=2) == EINVAL
+    assert bwd(scale=-1.0) == EINVAL
+    assert bwd(mask=3) == EINVAL
+    assert bwd(dq=None) == EINVAL
+    assert bwd(ws=None) == EINVAL
+    assert bwd(dq=P + 4) == EALIGN
+    assert bwd(strides=[64 * 256, 257, 128, 64 * 256, 256, 128, 64 * 256, 256, 128]) == EALIGN
+    assert bwd(Sq=4096, strides=[1 << 33, 1 << 21, 128, 64 * 256, 256, 128, 64 * 256, 256, 128]) == EUNSUPPORTED
+    assert bwd(B=0) == OK
+    assert lib.mhip_attn_bwd_workspace_bytes(2, 100, 64, 4, 2, 128) >= 2 * 2 * 4 * 100 * 4
+
+
+def test_elementwise_rejects(lib):
+    assert lib.mhip_flash_reduce(P, P, None, 8, 128, None) == EINVAL
+    assert lib.mhip_flash_reduce(P, P + 4, P, 8, 128, None) == EALIGN
+    assert lib.mhip_flash_reduce(P, P, P, -1, 128, None) == EINVAL
+    assert lib.mhip_flash_reduce(P, P, P, 0, 128, None) == OK
+    assert lib.mhip_tree_merge(P, None, P, 8, 128, 0, None) == EINVAL
+    assert lib.mhip_tree_merge(P + 8, P, P, 8, 128, 1, None) == EALIGN
+    assert lib.mhip_tree_merge(P, P, P, 0, 128, 1, None) == OK
+    assert lib.mhip_pack_reduce(None, P, P, None, 1, 8, 2, 128, None) == EINVAL
+    assert lib.mhip_pack_reduce(None, P, P, P, 0, 8, 2, 128, None) == OK
+    assert lib.mhip_grad_accumulate(None, P, None, 16, None) == EINVAL
+    assert lib.mhip_grad_accumulate(None, P + 2, P, 16, None) == EALIGN
+    assert lib.mhip_grad_accumulate(None, P, P, 0, None) == OK
