@@ -34,14 +34,10 @@ constexpr int kTileBytes = kBN * kD * 2;   // 16384: one K or V tile in LDS, 64 
 constexpr int kStages = 4;                 // K(t+1) .. K(t+4) and V(t) .. V(t+3) live while tile t is processed
 constexpr int kVBase = kStages * kTileBytes;
 constexpr int kOStride = kD + 8;   // epilogue staging of O, bf16 elements per row
-#ifndef MHIP_FWD_PINGPONG
-#define MHIP_FWD_PINGPONG 1
-#endif
 #ifndef MHIP_FWD_FRAG_DEPTH
 #define MHIP_FWD_FRAG_DEPTH 4
 #endif
 constexpr int kFragDepth = MHIP_FWD_FRAG_DEPTH;  // LDS operand reads in flight ahead of the MFMAs
-constexpr bool kPingPong = MHIP_FWD_PINGPONG;   // 0: all wavefronts run the phases in lock step
 
 struct FwdParams {
   const uint16_t* q; const uint16_t* k; const uint16_t* v;
@@ -90,7 +86,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
   const int lane = tid & 63;
   const int ln = lane & 31;
   const int hf = lane >> 5;
-  const bool group_b = wave >= 4;                 // second ping-pong group; these waves stage V
+  const bool group_b = wave >= 4;                 // second ping-pong group
 
   // ---- number of key tiles this Q tile has to visit -------------------------------------------
   int kv_end = p.Sc;
@@ -367,7 +363,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
   // (over K(t), last read in the matrix phase of tile t-1) and V(t+3) (over V(t-1)), and before the
   // barrier that ends the phase waits for the copies it started one tile earlier: those are then visible
   // to every wavefront two barriers later, in time for first_frags of K(t+3) and the matrix phase of V(t+2).
-  if (kPingPong && group_b) __builtin_amdgcn_s_barrier();
+  if (group_b) __builtin_amdgcn_s_barrier();
   for (int t = 0; t + 1 < ntiles; ++t) {
     // ---- matrix phase: S^T(t+1) = K(t+1) Q^T and O^T += V^T(t) P^T(t), first part of softmax(t+1) ------
     __builtin_amdgcn_s_setprio(2);
@@ -385,7 +381,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     __builtin_amdgcn_s_barrier();
   }
   if (ntiles > 0) pv((ntiles - 1) & 3);             // last tile: nothing left to prefetch or exponentiate
-  if (kPingPong && !group_b) __builtin_amdgcn_s_barrier();
+  if (!group_b) __builtin_amdgcn_s_barrier();
 
   // ---- epilogue -----------------------------------------------------------------------------------
   const float l_tot = pair_sum(l_run);
