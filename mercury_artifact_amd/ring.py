@@ -6,7 +6,10 @@ name (utils/flash_attn_dsl.py:127-180, 182-235, 237-291, 345-408; utils/attn_bwd
 neighbour exchange.  The body is the loop the code generator emits for that template
 (mercury/backend/pytorch/codegen.py:264-355, 443-523): take the current KV chunk, start the hop for
 the next one, run the block kernel through ``_flash_attn_forward(**params)``, fold with
-``update_out_and_lse``, and store after the last step.
+``update_out_and_lse``, and store after the last step.  By default the last merge writes ``o`` / ``lse``
+itself (``fused_epilogue=True``: the same arithmetic and bit-identical results, without the fp32 round trip
+of the merged accumulator through memory); ``fused_epilogue=False`` runs the generated code's literal
+sequence ``o[...] = _out.to(o.dtype)``, ``lse[...] = _lse.squeeze(-1).transpose(1, 2)``.
 """
 from __future__ import annotations
 
@@ -103,7 +106,7 @@ def _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, 
 
 def flash_attn_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False, window_size=(-1, -1),
                        alibi_slopes=None, deterministic=False, *, ring: LocalRing,
-                       fused_epilogue: bool = False):
+                       fused_epilogue: bool = True):
     """Single-ring forward step (template utils/flash_attn_dsl.py:127-180).  q (B,Sq,H,D), kv the
     rank's own (2,B,Sc,H,D), o (B,Sq,H,D) and lse (B,H,Sq) are written."""
     _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes, ring,
@@ -111,7 +114,7 @@ def flash_attn_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False, 
 
 
 def gqa_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False, window_size=(-1, -1),
-                alibi_slopes=None, deterministic=False, *, ring: LocalRing, fused_epilogue: bool = False):
+                alibi_slopes=None, deterministic=False, *, ring: LocalRing, fused_epilogue: bool = True):
     """GQA forward step (template utils/flash_attn_dsl.py:182-235): kv has Hkv heads, q has
     Hkv * HEADS_PER_GROUP; the block kernel maps q head h to kv head h // HEADS_PER_GROUP."""
     _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes, ring,
@@ -120,7 +123,7 @@ def gqa_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False, window_
 
 def flash_attn_pack_split_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False,
                              window_size=(-1, -1), alibi_slopes=None, deterministic=False, *,
-                             ring: LocalRing, fused_epilogue: bool = False):
+                             ring: LocalRing, fused_epilogue: bool = True):
     """Double-ring forward step (template utils/flash_attn_dsl.py:237-291): ``ring`` is built on the
     2-D mesh ``(inner, outer)``; the loop order and hops follow from the mesh shape."""
     if len(ring.mesh_shape) != 2:
@@ -250,7 +253,7 @@ def quantize_e4m3(x: torch.Tensor):
 
 def fp8_pack_split_kv(q, kv, o, lse, softmax_scale, q_descale, k_descale, v_descale, dropout_p=0,
                       causal=False, window_size=(-1, -1), alibi_slopes=None, deterministic=False, *,
-                      ring: LocalRing, fused_epilogue: bool = False):
+                      ring: LocalRing, fused_epilogue: bool = True):
     """Forward step on e4m3 Q/K/V with per-tensor descales (not in the reference); any mesh."""
     _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes, ring,
                   fused_epilogue, q_descale=q_descale, k_descale=k_descale, v_descale=v_descale)
