@@ -3,9 +3,10 @@
 
 Workload = the headline bf16 configuration: batch 1, 32 heads, head dim 128, local Q of 4096 rows, 8 KV chunks
 of 4096 rows (32768 keys), non-causal, N(0,1) inputs cast to bf16, softmax scale 128^-0.5.
-A step = 8 block-forward kernels + the first-call cast + 7 LSE merges, the last of which also writes the
-bf16 output and the (B,H,S) LSE (the drivers' default; the generated code's literal epilogue of separate
-torch copies is timed beside it), driven through the same operators Mercury's generated code calls.  Inputs are resident in HBM before
+A step = 8 block-forward kernels + ONE fold of the 8 block results into the bf16 output and the (B,H,S) LSE
+(the ring drivers' default: the fold is associative, so the chain of 7 LSE merges and the epilogue copies of
+the generated code collapse into one pass over the block outputs; that literal chain is timed beside it),
+driven through the same block operator Mercury's generated code calls.  Inputs are resident in HBM before
 the timed region.  Prints ONE JSON line.
 """
 from __future__ import annotations
@@ -145,7 +146,8 @@ def main() -> int:
 
     # per-kernel durations: HIP events on the stream the kernels are launched on (torch's current one), inside
     # the timed region.  An event pair costs a few microseconds of stream time, so each step brackets ONE of its
-    # forward launches and ONE of its plain merges (rotating through the chunks) instead of all 15.
+    # forward launches (rotating through the chunks) and the fold; the literal chain further down brackets ONE
+    # of its plain merges per step.
     fwd_events, merge_events = [], []
     real_fwd, real_merge = FI.attn_fwd_block, MG.merge_into
     recording = {"on": False, "step": 0, "fwd": 0, "merge": 0}
@@ -167,13 +169,29 @@ def main() -> int:
         return wrapper
 
     FI.attn_fwd_block = timed(real_fwd, fwd_events, "fwd", W, lambda a: True)
-    # plain merges only: the first call (a cast) and the last one (which also writes the bf16 output) move
-    # other byte counts
-    MG.merge_into = timed(real_merge, merge_events, "merge", W - 2, lambda a: a[0] is not None and a[4] is not None)
+    # plain merges only (they run in the literal chain timed further down): the first call is a cast
+    MG.merge_into = timed(real_merge, merge_events, "merge", W - 1, lambda a: a[0] is not None and a[4] is not None)
 
-    def step(fused=True):
+    many_events = []
+    real_many = MG.merge_many
+
+    def timed_many(*a, **kw):
+        if not recording["on"]:
+            return real_many(*a, **kw)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        r = real_many(*a, **kw)
+        e1.record()
+        many_events.append((e0, e1))
+        return r
+
+    from mercury_artifact_amd import ring as RG
+    RG.merge_many = timed_many
+
+    def step(literal=False):
         ring = M.LocalRing((W,), rank, kvs)
-        M.flash_attn_pack_kv(q, kvs[rank], o, lse, scale, ring=ring, fused_epilogue=fused)
+        M.flash_attn_pack_kv(q, kvs[rank], o, lse, scale, ring=ring, fused_epilogue=not literal,
+                             deferred_merge=not literal)
 
     for _ in range(args.warmup):
         step()
@@ -195,24 +213,31 @@ def main() -> int:
     fwd_ms = sum(e0.elapsed_time(e1) for e0, e1 in fwd_events) / max(len(fwd_events), 1)
     fwd_tflops = flops_per_block / (fwd_ms * 1e-3) / 1e12
     rows = B * Sq * H
+    many_bytes = rows * (W * (D * 2 + 4) + D * 2 + 4)
+    many_ms = sum(e0.elapsed_time(e1) for e0, e1 in many_events) / max(len(many_events), 1)
+    many_gbs = many_bytes / (many_ms * 1e-3) / 1e9
+
+    # the same step as the generated code spells it: update_out_and_lse after every chunk (the fp32
+    # accumulator read and written once per chunk), then the cast and the transposed copy of the epilogue.
+    # Also timed, with one plain merge per step bracketed by events.
+    for _ in range(2):
+        step(True)
+    torch.cuda.synchronize()
+    recording["on"] = True
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        recording.update(step=i, fwd=W + 1, merge=0)      # forward launches are not sampled again
+        step(True)
+    torch.cuda.synchronize()
+    unfused_ms = (time.perf_counter() - t0) / args.steps * 1e3
+    recording["on"] = False
     merge_bytes = rows * (D * 10 + 12)
     real_merges = merge_events
     merge_ms = sum(e0.elapsed_time(e1) for e0, e1 in real_merges) / max(len(real_merges), 1)
     merge_gbs = merge_bytes / (merge_ms * 1e-3) / 1e9
 
-    # the same step with the generated code's literal epilogue (fp32 accumulator written, then cast and
-    # transposed by separate torch copies): identical results, three more passes over the output
-    for _ in range(2):
-        step(False)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step(False)
-    torch.cuda.synchronize()
-    unfused_ms = (time.perf_counter() - t0) / args.steps * 1e3
-
     # the same step replayed as one HIP graph (one launch instead of ~25; identical kernels and results)
-    FI.attn_fwd_block, MG.merge_into = real_fwd, real_merge
+    FI.attn_fwd_block, MG.merge_into, RG.merge_many = real_fwd, real_merge, real_many
     graph_ms, graph_same = None, None
     try:
         graphed = M.GraphedStep(step)
@@ -253,14 +278,18 @@ def main() -> int:
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "headline bf16 configuration: non-causal MHA, B1 H32 D128, local Q 4096 x 8 KV chunks "
-                               "of 4096 (single ring, rank 0), 8 block forwards + 7 LSE merges, epilogue fused into the last merge",
+                               "of 4096 (single ring, rank 0), 8 block forwards + one fold of the 8 block results",
                    "flops_per_step": flops_per_step, "pct_of_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
-                   "literal_epilogue_ms_per_step": round(unfused_ms, 4),
+                   "literal_merge_chain_ms_per_step": round(unfused_ms, 4),
                    "hip_graph_ms_per_step": graph_ms, "hip_graph_bit_identical": graph_same,
                    "device": props.gcnArchName, "cus": props.multi_processor_count},
         "roofline": {"bound": "mfma", "kernel": "attn_fwd_bf16_d128", "achieved": round(fwd_tflops, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(fwd_tflops / PEAK_BF16_TFLOPS, 4),
                      "traffic": TRAFFIC_FWD_BYTES, "avg_launch_ms": round(fwd_ms, 4), "launches": len(fwd_events)},
+        "roofline_merge_many": {"bound": "hbm", "kernel": "lse_merge_many_kernel", "achieved": round(many_gbs, 1),
+                                "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(many_gbs / PEAK_HBM_GBS, 4),
+                                "traffic": None, "avg_launch_ms": round(many_ms, 5), "launches": len(many_events),
+                                "bytes_per_launch": many_bytes},
         "roofline_merge": {"bound": "hbm", "kernel": "lse_merge_kernel", "achieved": round(merge_gbs, 1),
                            "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(merge_gbs / PEAK_HBM_GBS, 4),
                            "traffic": TRAFFIC_MERGE_BYTES, "avg_launch_ms": round(merge_ms, 5), "launches": len(real_merges),

@@ -109,6 +109,23 @@ int mhip_lse_merge(const float* acc_out, const float* acc_lse,
                    void* stream);
 
 /*
+ * All block results of a ring step folded at once.  Replaces the chain of N update_out_and_lse calls of
+ * the chunk loop (utils/flash_attn_dsl.py:51-71, one per chunk) together with the stores of
+ * utils/flash_attn_dsl.py:178-179: with L = logsumexp_i(lse_i),
+ *   final_out = bf16(sum_i exp(lse_i - L) * out_i),  final_lse = L,
+ * which is what the chain computes (the fold is associative) without moving the fp32 accumulator through
+ * memory N - 1 times.  block_outs / block_lses are HOST arrays of n device pointers (1 <= n <= 16):
+ * block_outs[i] bf16 (B,Sq,Hq,D) addressed with the element strides bo_sb, bo_ss, bo_sh (multiples of 8,
+ * 16-byte aligned base, D contiguous), block_lses[i] fp32 (B,Hq,Sq) contiguous.  final_out bf16
+ * (B,Sq,Hq,D) contiguous, final_lse fp32 (B,Hq,Sq) contiguous.  D in {64, 128, 256}.  Rows whose lse is
+ * -inf in every block get (0, -inf).
+ */
+int mhip_lse_merge_many(const void* const* block_outs, const float* const* block_lses, int n,
+                        void* final_out, float* final_lse,
+                        int B, int Sq, int Hq, int D,
+                        int64_t bo_sb, int64_t bo_ss, int64_t bo_sh, void* stream);
+
+/*
  * Packed merge.  Replaces TorchScript `flash_reduce` (utils/flash_attn_dsl.py:293-305):
  * lhs, rhs, dst are contiguous fp32 (rows, D+1), 16-byte aligned; dst must not overlap lhs
  * or rhs (the reference's flash_reduce returns a new tensor as well).

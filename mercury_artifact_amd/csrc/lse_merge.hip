@@ -315,6 +315,81 @@ __global__ __launch_bounds__(256) void pack_reduce_kernel(const float* __restric
   }
 }
 
+// ---- all blocks of a step at once --------------------------------------------------------------------
+// The chunk loop of a ring step folds N block results into the accumulators one after the other
+// (utils/flash_attn_dsl.py:51-71 called once per chunk, then the stores of :178-179), which moves the fp32
+// accumulator through memory N - 1 times.  Folding is associative: with L = logsumexp_i(lse_i) the end
+// result is out = sum_i exp(lse_i - L) * out_i, lse = L.  This kernel reads the N bf16 block outputs once
+// and writes the bf16 output and the (B,H,S) LSE directly.  Rows whose lse is -inf everywhere give
+// (0, -inf).  One row = D/8 lanes x 8 contiguous head-dim values (16 bytes of bf16), ROWS rows per thread.
+constexpr int kMaxBlocks = 16;
+struct MergeManyParams {
+  const uint16_t* out[kMaxBlocks];
+  const float* lse[kMaxBlocks];
+  uint16_t* final_out; float* final_lse;
+  int n, Sq, Hq;
+  int64_t rows;
+  int64_t bo_sb, bo_ss, bo_sh;
+};
+
+template <int LPR, int N>          // N = 0: run-time block count
+__global__ __launch_bounds__(256) void lse_merge_many_kernel(const MergeManyParams p) {
+  constexpr int D = LPR * 8;
+  constexpr int kRowsPerPass = 256 / LPR;
+  const int n = N > 0 ? N : p.n;
+  const int64_t row = (int64_t)blockIdx.x * kRowsPerPass + threadIdx.x / LPR;
+  if (row >= p.rows) return;
+  const int col = (threadIdx.x % LPR) * 8;
+  const uint32_t h = (uint32_t)row % (uint32_t)p.Hq;
+  const uint32_t bs = (uint32_t)row / (uint32_t)p.Hq;
+  const uint32_t s = bs % (uint32_t)p.Sq;
+  const uint32_t b = bs / (uint32_t)p.Sq;
+  const int64_t o_off = b * p.bo_sb + s * p.bo_ss + h * p.bo_sh + col;
+  const int64_t l_off = ((int64_t)b * p.Hq + h) * p.Sq + s;
+  u32x4 blk[N > 0 ? N : kMaxBlocks];
+  float l[N > 0 ? N : kMaxBlocks];
+#pragma unroll
+  for (int i = 0; i < (N > 0 ? N : kMaxBlocks); ++i) {
+    if (i < n) {
+      blk[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.out[i] + o_off));
+      l[i] = p.lse[i][l_off];
+    }
+  }
+  float m = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < (N > 0 ? N : kMaxBlocks); ++i)
+    if (i < n) m = fmaxf(m, l[i]);
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < (N > 0 ? N : kMaxBlocks); ++i) {
+    if (i < n) {
+      const float w = (m == -INFINITY) ? 0.f : __expf(l[i] - m);
+      sum += w;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc[2 * j] = __builtin_fmaf(w, bf16_lo(blk[i][j]), acc[2 * j]);
+        acc[2 * j + 1] = __builtin_fmaf(w, bf16_hi(blk[i][j]), acc[2 * j + 1]);
+      }
+    }
+  }
+  const float inv = sum > 0.f ? 1.f / sum : 0.f;
+  u32x4 w4;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) w4[j] = pack_bf16(acc[2 * j] * inv, acc[2 * j + 1] * inv);
+  *reinterpret_cast<u32x4*>(p.final_out + row * D + col) = w4;
+  if (col == 0) p.final_lse[l_off] = sum > 0.f ? m + __logf(sum) : -INFINITY;
+}
+
+template <int LPR>
+void launch_merge_many(const MergeManyParams& p, hipStream_t st) {
+  constexpr int kRowsPerPass = 256 / LPR;
+  const dim3 grid((unsigned)((p.rows + kRowsPerPass - 1) / kRowsPerPass)), block(256);
+  if (p.n == 8) hipLaunchKernelGGL((lse_merge_many_kernel<LPR, 8>), grid, block, 0, st, p);
+  else if (p.n == 4) hipLaunchKernelGGL((lse_merge_many_kernel<LPR, 4>), grid, block, 0, st, p);
+  else hipLaunchKernelGGL((lse_merge_many_kernel<LPR, 0>), grid, block, 0, st, p);
+}
+
 template <bool HAS_ACC>
 __global__ __launch_bounds__(256) void grad_accumulate_kernel(const float* acc, const uint16_t* block,
                                                               float* dst, int64_t n) {
@@ -396,6 +471,38 @@ extern "C" int mhip_lse_merge(const float* acc_out, const float* acc_lse,
     else if (first) hipLaunchKernelGGL((lse_merge_generic<true, false>), grid, block, 0, st, p, D);
     else if (fin) hipLaunchKernelGGL((lse_merge_generic<false, true>), grid, block, 0, st, p, D);
     else hipLaunchKernelGGL((lse_merge_generic<false, false>), grid, block, 0, st, p, D);
+  }
+  return launch_status();
+}
+
+extern "C" int mhip_lse_merge_many(const void* const* block_outs, const float* const* block_lses, int n,
+                                   void* final_out, float* final_lse,
+                                   int B, int Sq, int Hq, int D,
+                                   int64_t bo_sb, int64_t bo_ss, int64_t bo_sh, void* stream) {
+  if (B < 0 || Sq < 0 || Hq < 0 || D <= 0 || n < 1 || n > kMaxBlocks) return MHIP_EINVAL;
+  if (D != 64 && D != 128 && D != 256) return MHIP_EUNSUPPORTED;
+  const int64_t rows = (int64_t)B * Sq * Hq;
+  if (rows == 0) return MHIP_OK;
+  if (rows >= (int64_t(1) << 31)) return MHIP_EUNSUPPORTED;
+  if (!block_outs || !block_lses || !final_out || !final_lse) return MHIP_EINVAL;
+  if ((bo_sb & 7) || (bo_ss & 7) || (bo_sh & 7)) return MHIP_EALIGN;
+  if (!aligned16(final_out)) return MHIP_EALIGN;
+  MergeManyParams p;
+  for (int i = 0; i < kMaxBlocks; ++i) { p.out[i] = nullptr; p.lse[i] = nullptr; }
+  for (int i = 0; i < n; ++i) {
+    if (!block_outs[i] || !block_lses[i]) return MHIP_EINVAL;
+    if (!aligned16(block_outs[i])) return MHIP_EALIGN;
+    p.out[i] = static_cast<const uint16_t*>(block_outs[i]);
+    p.lse[i] = block_lses[i];
+  }
+  p.final_out = static_cast<uint16_t*>(final_out); p.final_lse = final_lse;
+  p.n = n; p.Sq = Sq; p.Hq = Hq; p.rows = rows;
+  p.bo_sb = bo_sb; p.bo_ss = bo_ss; p.bo_sh = bo_sh;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  switch (D) {
+    case 64: launch_merge_many<8>(p, st); break;
+    case 128: launch_merge_many<16>(p, st); break;
+    default: launch_merge_many<32>(p, st); break;
   }
   return launch_status();
 }

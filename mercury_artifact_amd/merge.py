@@ -15,7 +15,7 @@ import torch
 from . import _native as N
 
 __all__ = ["get_default_args", "update_out_and_lse", "_update_out_and_lse", "flash_reduce",
-           "pack_block", "merge_into", "grad_accumulate", "update_out_and_lse_collective", "add_collective",
+           "pack_block", "merge_into", "merge_many", "grad_accumulate", "update_out_and_lse_collective", "add_collective",
            "LocalGroup"]
 
 
@@ -81,6 +81,41 @@ def merge_into(acc_out: Optional[torch.Tensor], acc_lse: Optional[torch.Tensor],
             *(z3 if dst_lse is None else _row_strides(dst_lse)),
             N.stream_of(block_out))
     N.check(code, "mhip_lse_merge")
+
+
+MAX_MERGE_MANY = 16
+
+
+def merge_many(block_outs: Sequence[torch.Tensor], block_lses: Sequence[torch.Tensor],
+               final_out: torch.Tensor, final_lse: torch.Tensor) -> None:
+    """All block results of a step folded by one call of mhip_lse_merge_many: what the chain of
+    ``update_out_and_lse`` calls of the chunk loop plus the stores of utils/flash_attn_dsl.py:178-179
+    compute (the fold is associative), reading every bf16 block output once.  block_outs[i] (B,Sq,Hq,D)
+    bf16 with one set of strides, block_lses[i] (B,Hq,Sq) fp32 contiguous, at most ``MAX_MERGE_MANY``
+    blocks; final_out (B,Sq,Hq,D) bf16 and final_lse (B,Hq,Sq) fp32, both contiguous, are written."""
+    import ctypes
+
+    n = len(block_outs)
+    if n != len(block_lses) or not 1 <= n <= MAX_MERGE_MANY:
+        raise RuntimeError(f"merge_many takes 1..{MAX_MERGE_MANY} blocks with one lse each")
+    N.require_cuda(*block_outs, *block_lses, final_out, final_lse)
+    B, Sq, Hq, D = block_outs[0].shape
+    strides = block_outs[0].stride()
+    for bo, bl in zip(block_outs, block_lses):
+        if bo.shape != (B, Sq, Hq, D) or bo.dtype != torch.bfloat16 or bo.stride() != strides or strides[-1] != 1:
+            raise RuntimeError("block outputs must be bfloat16 (B,Sq,Hq,D) with one set of strides")
+        if bl.shape != (B, Hq, Sq) or bl.dtype != torch.float32 or not bl.is_contiguous():
+            raise RuntimeError("block lse must be contiguous float32 (B,Hq,Sq)")
+    if final_out.shape != (B, Sq, Hq, D) or final_out.dtype != torch.bfloat16 or not final_out.is_contiguous():
+        raise RuntimeError("final_out must be contiguous bfloat16 (B,Sq,Hq,D)")
+    if final_lse.shape != (B, Hq, Sq) or final_lse.dtype != torch.float32 or not final_lse.is_contiguous():
+        raise RuntimeError("final_lse must be contiguous float32 (B,Hq,Sq)")
+    outs = (ctypes.c_void_p * n)(*[t.data_ptr() for t in block_outs])
+    lses = (ctypes.c_void_p * n)(*[t.data_ptr() for t in block_lses])
+    with torch.cuda.device(final_out.device):
+        code = N.lib().mhip_lse_merge_many(outs, lses, n, N.ptr(final_out), N.ptr(final_lse), B, Sq, Hq, D,
+                                           strides[0], strides[1], strides[2], N.stream_of(final_out))
+    N.check(code, "mhip_lse_merge_many")
 
 
 def _update_out_and_lse(out: torch.Tensor, lse: torch.Tensor, block_out: torch.Tensor,

@@ -6,10 +6,16 @@ name (utils/flash_attn_dsl.py:127-180, 182-235, 237-291, 345-408; utils/attn_bwd
 neighbour exchange.  The body is the loop the code generator emits for that template
 (mercury/backend/pytorch/codegen.py:264-355, 443-523): take the current KV chunk, start the hop for
 the next one, run the block kernel through ``_flash_attn_forward(**params)``, fold with
-``update_out_and_lse``, and store after the last step.  By default the last merge writes ``o`` / ``lse``
-itself (``fused_epilogue=True``: the same arithmetic and bit-identical results, without the fp32 round trip
-of the merged accumulator through memory); ``fused_epilogue=False`` runs the generated code's literal
-sequence ``o[...] = _out.to(o.dtype)``, ``lse[...] = _lse.squeeze(-1).transpose(1, 2)``.
+``update_out_and_lse``, and store after the last step.
+
+Two defaults of the forward drivers depart from the literal sequence without changing what is computed:
+``deferred_merge=True`` keeps the bf16 block results of all chunks and folds them with ONE
+``merge_many`` call after the last chunk (the fold is associative; every block output is read once
+instead of the fp32 accumulator travelling through memory once per chunk; results agree with the chain
+to fp32 rounding), and ``fused_epilogue=True`` lets the last merge of the chain write ``o`` / ``lse``
+itself (bit-identical).  ``deferred_merge=False, fused_epilogue=False`` is the generated code's literal
+sequence: ``update_out_and_lse`` per chunk, then ``o[...] = _out.to(o.dtype)``,
+``lse[...] = _lse.squeeze(-1).transpose(1, 2)``.
 """
 from __future__ import annotations
 
@@ -18,7 +24,8 @@ from typing import Optional
 import torch
 
 from .flash_attn_interface import _flash_attn_backward, _flash_attn_forward
-from .merge import get_default_args, grad_accumulate, merge_into, pack_block, update_out_and_lse
+from .merge import (MAX_MERGE_MANY, get_default_args, grad_accumulate, merge_into, merge_many, pack_block,
+                    update_out_and_lse)
 from .schedule import (LocalRing, n_dim_to_one_dim, one_dim_to_n_dim, reduce_buffer_route, shift_tuple_element,
                        zigzag_step)
 
@@ -73,12 +80,15 @@ def _fwd_params(q, k, v, softmax_scale, dropout_p, causal, window_size, alibi_sl
 
 
 def _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes,
-                  ring: LocalRing, fused_epilogue: bool, **extra):
+                  ring: LocalRing, fused_epilogue: bool, deferred_merge: bool, **extra):
+    blocks = []
     _out = None
     _lse = None
     _kv = None
     _next_kv = None
     steps = list(_hops(ring))
+    defer = (deferred_merge and len(steps) <= MAX_MERGE_MANY and o.dtype == torch.bfloat16
+             and o.is_contiguous() and lse.is_contiguous())
     for step, hop in enumerate(steps):
         if step == 0:
             _kv = kv.contiguous()
@@ -95,6 +105,12 @@ def _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, 
                                                     window_size, alibi_slopes, **extra))
         assert len(outputs) == 4
         block_out, block_lse, _, _ = outputs
+        if defer:
+            blocks.append((block_out, block_lse))
+            if step + 1 == len(steps):
+                merge_many([b[0] for b in blocks], [b[1] for b in blocks], o, lse)
+                return
+            continue
         if fused_epilogue and step + 1 == len(steps):
             # last merge writes o / lse directly (same arithmetic, two passes fewer)
             merge_into(_out, _lse, block_out, block_lse, None, None, o, lse)
@@ -106,30 +122,31 @@ def _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, 
 
 def flash_attn_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False, window_size=(-1, -1),
                        alibi_slopes=None, deterministic=False, *, ring: LocalRing,
-                       fused_epilogue: bool = True):
+                       fused_epilogue: bool = True, deferred_merge: bool = True):
     """Single-ring forward step (template utils/flash_attn_dsl.py:127-180).  q (B,Sq,H,D), kv the
     rank's own (2,B,Sc,H,D), o (B,Sq,H,D) and lse (B,H,Sq) are written."""
     _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes, ring,
-                  fused_epilogue)
+                  fused_epilogue, deferred_merge)
 
 
 def gqa_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False, window_size=(-1, -1),
-                alibi_slopes=None, deterministic=False, *, ring: LocalRing, fused_epilogue: bool = True):
+                alibi_slopes=None, deterministic=False, *, ring: LocalRing, fused_epilogue: bool = True,
+                deferred_merge: bool = True):
     """GQA forward step (template utils/flash_attn_dsl.py:182-235): kv has Hkv heads, q has
     Hkv * HEADS_PER_GROUP; the block kernel maps q head h to kv head h // HEADS_PER_GROUP."""
     _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes, ring,
-                  fused_epilogue)
+                  fused_epilogue, deferred_merge)
 
 
 def flash_attn_pack_split_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False,
                              window_size=(-1, -1), alibi_slopes=None, deterministic=False, *,
-                             ring: LocalRing, fused_epilogue: bool = True):
+                             ring: LocalRing, fused_epilogue: bool = True, deferred_merge: bool = True):
     """Double-ring forward step (template utils/flash_attn_dsl.py:237-291): ``ring`` is built on the
     2-D mesh ``(inner, outer)``; the loop order and hops follow from the mesh shape."""
     if len(ring.mesh_shape) != 2:
         raise ValueError("the double ring needs a 2-D mesh (inner, outer)")
     _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes, ring,
-                  fused_epilogue)
+                  fused_epilogue, deferred_merge)
 
 
 def flash_attn_expose_reduce(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False,
@@ -253,10 +270,10 @@ def quantize_e4m3(x: torch.Tensor):
 
 def fp8_pack_split_kv(q, kv, o, lse, softmax_scale, q_descale, k_descale, v_descale, dropout_p=0,
                       causal=False, window_size=(-1, -1), alibi_slopes=None, deterministic=False, *,
-                      ring: LocalRing, fused_epilogue: bool = True):
+                      ring: LocalRing, fused_epilogue: bool = True, deferred_merge: bool = True):
     """Forward step on e4m3 Q/K/V with per-tensor descales (not in the reference); any mesh."""
     _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes, ring,
-                  fused_epilogue, q_descale=q_descale, k_descale=k_descale, v_descale=v_descale)
+                  fused_epilogue, deferred_merge, q_descale=q_descale, k_descale=k_descale, v_descale=v_descale)
 
 
 def flash_attn_backward(q, kv, o, lse, dout, dq, dkv, softmax_scale, dropout_p=0, causal=False,

@@ -32,7 +32,7 @@ import torch
 
 __all__ = [
     "block_attention", "single_pass_attention", "merge_reference", "merge_closed_form",
-    "update_out_and_lse", "pack_block", "flash_reduce", "tree_merge", "block_backward",
+    "update_out_and_lse", "merge_chain", "pack_block", "flash_reduce", "tree_merge", "block_backward",
     "single_ring_order", "double_ring_order", "ring_divide_order",
     "zigzag_blocks", "zigzag_step", "zigzag_local_positions",
     "quantize_e4m3", "dequantize",
@@ -132,6 +132,16 @@ def update_out_and_lse(out, lse, block_out, block_lse, slice_=None, merge=merge_
     else:
         out, lse = merge(out, lse, block_out, block_lse)
     return out, lse
+
+
+def merge_chain(block_outs, block_lses, acc_dtype=torch.float64):
+    """The chunk loop's chain of ``update_out_and_lse`` calls over all block results followed by the
+    stores of utils/flash_attn_dsl.py:178-179: returns ``(out (B,Sq,Hq,D), lse (B,Hq,Sq))`` in
+    ``acc_dtype``.  Built from the pinned pieces above; what a one-pass fold of all blocks has to equal."""
+    out = lse = None
+    for bo, bl in zip(block_outs, block_lses):
+        out, lse = update_out_and_lse(out, lse, bo, bl, acc_dtype=acc_dtype)
+    return out, lse.squeeze(dim=-1).transpose(1, 2)
 
 
 def pack_block(block_out, block_lse):

@@ -8,8 +8,8 @@ import torch
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("fused", [False, True])
-def test_graphed_single_ring_step_matches_eager(fused):
+@pytest.mark.parametrize("fused,deferred", [(False, False), (True, False), (True, True)])
+def test_graphed_single_ring_step_matches_eager(fused, deferred):
     import mercury_artifact_amd as M
 
     B, S, H, D, W, rank = 2, 256, 4, 128, 4, 1
@@ -22,7 +22,7 @@ def test_graphed_single_ring_step_matches_eager(fused):
 
     def step():
         M.flash_attn_pack_kv(q, chunks[rank], o, lse, scale, ring=M.LocalRing((W,), rank, chunks),
-                             fused_epilogue=fused)
+                             fused_epilogue=fused, deferred_merge=deferred)
 
     graphed = M.GraphedStep(step)
     for it in range(4):

@@ -177,3 +177,62 @@ def test_add_collective_sums_the_group():
     assert torch.allclose(mine, peers[0] + peers[1] + peers[2], atol=1e-6)
     with pytest.raises(ValueError):
         M.add_collective(mine, "reduce", M.LocalGroup(peers, rank=0))
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 8, 16])
+@pytest.mark.parametrize("B,Sq,H,D", [(2, 37, 3, 128), (1, 64, 4, 64), (1, 9, 2, 256)])
+def test_merge_many_matches_the_chain(n, B, Sq, H, D):
+    """One fold of all block results against the chain of reference merges in fp64 followed by the
+    epilogue.  The output is bf16: atol 1e-3 + rtol 2^-8 (one bf16 rounding of the result); lse 1e-5."""
+    import mercury_artifact_amd as M
+
+    print(f"merge_many case n={n} {B} {Sq} {H} {D}", flush=True)
+    g = torch.Generator().manual_seed(100 + n)
+    outs = [torch.randn(B, Sq, H, D, generator=g).bfloat16() for _ in range(n)]
+    lses = [torch.randn(B, H, Sq, generator=g) * 3 + 5 for _ in range(n)]
+    # rows that are -inf in one block, in all but one, and in every block
+    lses[0][0, 0, 0] = -math.inf
+    if n == 1:
+        outs[0][0, 0, 0] = 0           # a lone block's -inf row carries out = 0, as the block kernel writes it
+    for i in range(1, n):
+        lses[i][0, 0, 1] = -math.inf
+    for i in range(n):
+        lses[i][0, 0, 2] = -math.inf
+        outs[i][0, 2, 0] = 0
+    ro, rl = O.merge_chain(outs, lses)
+    fo = torch.full((B, Sq, H, D), 7.0, dtype=torch.bfloat16, device="cuda")
+    fl = torch.full((B, H, Sq), 7.0, dtype=torch.float32, device="cuda")
+    M.merge_many([t.cuda() for t in outs], [t.cuda() for t in lses], fo, fl)
+    fo, fl = fo.float().cpu(), fl.cpu()
+    # the all -inf row: the chain NaNs (so does the reference), the kernel gives (0, -inf)
+    assert torch.equal(fo[0, 2, 0], torch.zeros(D)) and fl[0, 0, 2].item() == -math.inf
+    ro[0, 2, 0], rl[0, 0, 2] = 0, -math.inf
+    assert not torch.isnan(fo).any() and not torch.isnan(fl).any()
+    assert ((fo - ro.float()).abs() - (1e-3 + 2 ** -8 * ro.float().abs())).max().item() <= 0
+    finite = torch.isfinite(rl)
+    assert torch.equal(torch.isfinite(fl), finite)
+    assert ((fl[finite] - rl[finite].float()).abs() / rl[finite].float().abs().clamp_min(1.0)).max().item() <= 1e-5
+
+
+def test_merge_many_strided_blocks_and_errors():
+    import mercury_artifact_amd as M
+
+    B, Sq, H, D, n = 1, 50, 3, 128, 4
+    g = torch.Generator().manual_seed(5)
+    big = [torch.randn(B, Sq, 2 * H, D, generator=g).bfloat16().cuda() for _ in range(n)]
+    outs = [t[:, :, H:] for t in big]                       # head-sliced views: same strides, offset base
+    lses = [(torch.randn(B, H, Sq, generator=g) * 2).cuda() for _ in range(n)]
+    ro, rl = O.merge_chain([t.cpu() for t in outs], [t.cpu() for t in lses])
+    fo = torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device="cuda")
+    fl = torch.empty(B, H, Sq, dtype=torch.float32, device="cuda")
+    M.merge_many(outs, lses, fo, fl)
+    assert ((fo.float().cpu() - ro.float()).abs() - (1e-3 + 2 ** -8 * ro.float().abs())).max().item() <= 0
+    assert torch.allclose(fl.cpu(), rl.float(), atol=1e-5, rtol=1e-5)
+    with pytest.raises(RuntimeError):
+        M.merge_many(outs * 5, lses * 5, fo, fl)             # 20 blocks
+    with pytest.raises(RuntimeError):
+        M.merge_many(outs, lses[:-1], fo, fl)
+    with pytest.raises(RuntimeError):
+        M.merge_many([outs[0], big[1][:, :, :H].float()], lses[:2], fo, fl)
+    with pytest.raises(RuntimeError):
+        M.merge_many([t.cpu() for t in outs], lses, fo, fl)

@@ -32,8 +32,8 @@ def _compare(o, lse, ro, rl, out_atol=2e-2, lse_rtol=1e-3, rel_l2=1e-2):
 
 
 @pytest.mark.parametrize("rank", [0, 5])
-@pytest.mark.parametrize("fused", [False, True])
-def test_single_ring_reference_test_shape(rank, fused):
+@pytest.mark.parametrize("fused,deferred", [(False, False), (True, False), (True, True)])
+def test_single_ring_reference_test_shape(rank, fused, deferred):
     """B4 S4096 H5 D128 on an 8-rank ring (tests/test_ring_attn_codegen.py:84-87), one rank."""
     import mercury_artifact_amd as M
 
@@ -50,7 +50,7 @@ def test_single_ring_reference_test_shape(rank, fused):
     o = torch.empty_like(qd)
     lse = torch.empty(B, H, S // W, dtype=torch.float32, device="cuda")
     q_before, kv_before = qd.clone(), dev_kvs[rank].clone()
-    M.flash_attn_pack_kv(qd, dev_kvs[rank], o, lse, scale, ring=ring, fused_epilogue=fused)
+    M.flash_attn_pack_kv(qd, dev_kvs[rank], o, lse, scale, ring=ring, fused_epilogue=fused, deferred_merge=deferred)
     torch.cuda.synchronize()
     _compare(o, lse, ring_o, ring_l)
     assert (o.float().cpu() - ro).abs().max().item() < 1e-2 and (lse.cpu() - rl).abs().max().item() < 1e-2
