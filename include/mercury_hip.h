@@ -114,16 +114,19 @@ int mhip_lse_merge(const float* acc_out, const float* acc_lse,
  * utils/flash_attn_dsl.py:178-179: with L = logsumexp_i(lse_i),
  *   final_out = bf16(sum_i exp(lse_i - L) * out_i),  final_lse = L,
  * which is what the chain computes (the fold is associative) without moving the fp32 accumulator through
- * memory N - 1 times.  block_outs / block_lses are HOST arrays of n device pointers (1 <= n <= 16):
- * block_outs[i] bf16 (B,Sq,Hq,D) addressed with the element strides bo_sb, bo_ss, bo_sh (multiples of 8,
- * 16-byte aligned base, D contiguous), block_lses[i] fp32 (B,Hq,Sq) contiguous.  final_out bf16
- * (B,Sq,Hq,D) contiguous, final_lse fp32 (B,Hq,Sq) contiguous.  D in {64, 128, 256}.  Rows whose lse is
- * -inf in every block get (0, -inf).
+ * memory N - 1 times.  block_outs / block_lses / bo_sb / s_begin are HOST arrays of n entries
+ * (1 <= n <= 16; s_begin may be NULL = all zero).  Block i covers the sequence rows s >= s_begin[i]
+ * (rows before count as lse = -inf: the "second half of the Q rows" steps of a zigzag schedule):
+ * block_outs[i] bf16 (B, Sq - s_begin[i], Hq, D) addressed with the element strides bo_sb[i], bo_ss, bo_sh
+ * (multiples of 8, 16-byte aligned base, D contiguous), block_lses[i] fp32 (B, Hq, Sq - s_begin[i])
+ * contiguous.  final_out bf16 (B,Sq,Hq,D) contiguous, final_lse fp32 (B,Hq,Sq) contiguous.
+ * D in {64, 128, 256}.  Rows whose lse is -inf in every block get (0, -inf).
  */
-int mhip_lse_merge_many(const void* const* block_outs, const float* const* block_lses, int n,
+int mhip_lse_merge_many(const void* const* block_outs, const float* const* block_lses,
+                        const int64_t* bo_sb, const int* s_begin, int n,
                         void* final_out, float* final_lse,
                         int B, int Sq, int Hq, int D,
-                        int64_t bo_sb, int64_t bo_ss, int64_t bo_sh, void* stream);
+                        int64_t bo_ss, int64_t bo_sh, void* stream);
 
 /*
  * Packed merge.  Replaces TorchScript `flash_reduce` (utils/flash_attn_dsl.py:293-305):

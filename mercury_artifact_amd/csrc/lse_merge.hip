@@ -321,15 +321,19 @@ __global__ __launch_bounds__(256) void pack_reduce_kernel(const float* __restric
 // accumulator through memory N - 1 times.  Folding is associative: with L = logsumexp_i(lse_i) the end
 // result is out = sum_i exp(lse_i - L) * out_i, lse = L.  This kernel reads the N bf16 block outputs once
 // and writes the bf16 output and the (B,H,S) LSE directly.  Rows whose lse is -inf everywhere give
-// (0, -inf).  One row = D/8 lanes x 8 contiguous head-dim values (16 bytes of bf16), ROWS rows per thread.
+// (0, -inf).  A block may cover only the rows s >= s_begin[i] of the sequence dimension (the zigzag
+// schedule's "second half of the Q rows" steps); the rows before count as lse = -inf.
+// One row = D/8 lanes x 8 contiguous head-dim values (16 bytes of bf16) per thread.
 constexpr int kMaxBlocks = 16;
 struct MergeManyParams {
   const uint16_t* out[kMaxBlocks];
   const float* lse[kMaxBlocks];
   uint16_t* final_out; float* final_lse;
+  int s_begin[kMaxBlocks];        // first sequence row the block covers
+  int64_t bo_sb[kMaxBlocks];      // batch stride of the block's output, elements
   int n, Sq, Hq;
   int64_t rows;
-  int64_t bo_sb, bo_ss, bo_sh;
+  int64_t bo_ss, bo_sh;
 };
 
 template <int LPR, int N>          // N = 0: run-time block count
@@ -344,15 +348,20 @@ __global__ __launch_bounds__(256) void lse_merge_many_kernel(const MergeManyPara
   const uint32_t bs = (uint32_t)row / (uint32_t)p.Hq;
   const uint32_t s = bs % (uint32_t)p.Sq;
   const uint32_t b = bs / (uint32_t)p.Sq;
-  const int64_t o_off = b * p.bo_sb + s * p.bo_ss + h * p.bo_sh + col;
   const int64_t l_off = ((int64_t)b * p.Hq + h) * p.Sq + s;
   u32x4 blk[N > 0 ? N : kMaxBlocks];
   float l[N > 0 ? N : kMaxBlocks];
 #pragma unroll
   for (int i = 0; i < (N > 0 ? N : kMaxBlocks); ++i) {
     if (i < n) {
-      blk[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.out[i] + o_off));
-      l[i] = p.lse[i][l_off];
+      const int sb = p.s_begin[i];
+      l[i] = -INFINITY;
+      blk[i] = u32x4{0u, 0u, 0u, 0u};
+      if ((int)s >= sb) {
+        const int64_t o_off = b * p.bo_sb[i] + (int64_t)(s - sb) * p.bo_ss + h * p.bo_sh + col;
+        blk[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.out[i] + o_off));
+        l[i] = p.lse[i][((int64_t)b * p.Hq + h) * (p.Sq - sb) + (s - sb)];
+      }
     }
   }
   float m = -INFINITY;
@@ -475,29 +484,34 @@ extern "C" int mhip_lse_merge(const float* acc_out, const float* acc_lse,
   return launch_status();
 }
 
-extern "C" int mhip_lse_merge_many(const void* const* block_outs, const float* const* block_lses, int n,
+extern "C" int mhip_lse_merge_many(const void* const* block_outs, const float* const* block_lses,
+                                   const int64_t* bo_sb, const int* s_begin, int n,
                                    void* final_out, float* final_lse,
                                    int B, int Sq, int Hq, int D,
-                                   int64_t bo_sb, int64_t bo_ss, int64_t bo_sh, void* stream) {
+                                   int64_t bo_ss, int64_t bo_sh, void* stream) {
   if (B < 0 || Sq < 0 || Hq < 0 || D <= 0 || n < 1 || n > kMaxBlocks) return MHIP_EINVAL;
   if (D != 64 && D != 128 && D != 256) return MHIP_EUNSUPPORTED;
   const int64_t rows = (int64_t)B * Sq * Hq;
   if (rows == 0) return MHIP_OK;
   if (rows >= (int64_t(1) << 31)) return MHIP_EUNSUPPORTED;
-  if (!block_outs || !block_lses || !final_out || !final_lse) return MHIP_EINVAL;
-  if ((bo_sb & 7) || (bo_ss & 7) || (bo_sh & 7)) return MHIP_EALIGN;
+  if (!block_outs || !block_lses || !bo_sb || !final_out || !final_lse) return MHIP_EINVAL;
+  if ((bo_ss & 7) || (bo_sh & 7)) return MHIP_EALIGN;
   if (!aligned16(final_out)) return MHIP_EALIGN;
   MergeManyParams p;
-  for (int i = 0; i < kMaxBlocks; ++i) { p.out[i] = nullptr; p.lse[i] = nullptr; }
+  for (int i = 0; i < kMaxBlocks; ++i) { p.out[i] = nullptr; p.lse[i] = nullptr; p.s_begin[i] = 0; p.bo_sb[i] = 0; }
   for (int i = 0; i < n; ++i) {
     if (!block_outs[i] || !block_lses[i]) return MHIP_EINVAL;
-    if (!aligned16(block_outs[i])) return MHIP_EALIGN;
+    const int sb = s_begin ? s_begin[i] : 0;
+    if (sb < 0 || sb > Sq) return MHIP_EINVAL;
+    if (!aligned16(block_outs[i]) || (bo_sb[i] & 7)) return MHIP_EALIGN;
+    p.s_begin[i] = sb;
+    p.bo_sb[i] = bo_sb[i];
     p.out[i] = static_cast<const uint16_t*>(block_outs[i]);
     p.lse[i] = block_lses[i];
   }
   p.final_out = static_cast<uint16_t*>(final_out); p.final_lse = final_lse;
   p.n = n; p.Sq = Sq; p.Hq = Hq; p.rows = rows;
-  p.bo_sb = bo_sb; p.bo_ss = bo_ss; p.bo_sh = bo_sh;
+  p.bo_ss = bo_ss; p.bo_sh = bo_sh;
   hipStream_t st = static_cast<hipStream_t>(stream);
   switch (D) {
     case 64: launch_merge_many<8>(p, st); break;

@@ -87,34 +87,46 @@ MAX_MERGE_MANY = 16
 
 
 def merge_many(block_outs: Sequence[torch.Tensor], block_lses: Sequence[torch.Tensor],
-               final_out: torch.Tensor, final_lse: torch.Tensor) -> None:
+               final_out: torch.Tensor, final_lse: torch.Tensor,
+               row_begin: Optional[Sequence[int]] = None) -> None:
     """All block results of a step folded by one call of mhip_lse_merge_many: what the chain of
     ``update_out_and_lse`` calls of the chunk loop plus the stores of utils/flash_attn_dsl.py:178-179
-    compute (the fold is associative), reading every bf16 block output once.  block_outs[i] (B,Sq,Hq,D)
-    bf16 with one set of strides, block_lses[i] (B,Hq,Sq) fp32 contiguous, at most ``MAX_MERGE_MANY``
-    blocks; final_out (B,Sq,Hq,D) bf16 and final_lse (B,Hq,Sq) fp32, both contiguous, are written."""
+    compute (the fold is associative), reading every bf16 block output once.  Block i covers the sequence
+    rows ``row_begin[i]:`` (default 0, i.e. all rows; the ``slice_`` merges of a zigzag schedule pass the
+    start of their row range): block_outs[i] (B, Sq - row_begin[i], Hq, D) bf16 with contiguous heads,
+    block_lses[i] (B, Hq, Sq - row_begin[i]) fp32 contiguous, at most ``MAX_MERGE_MANY`` blocks;
+    final_out (B,Sq,Hq,D) bf16 and final_lse (B,Hq,Sq) fp32, both contiguous, are written."""
     import ctypes
 
     n = len(block_outs)
     if n != len(block_lses) or not 1 <= n <= MAX_MERGE_MANY:
         raise RuntimeError(f"merge_many takes 1..{MAX_MERGE_MANY} blocks with one lse each")
+    begins = [0] * n if row_begin is None else [int(x) for x in row_begin]
+    if len(begins) != n:
+        raise RuntimeError("row_begin needs one entry per block")
     N.require_cuda(*block_outs, *block_lses, final_out, final_lse)
-    B, Sq, Hq, D = block_outs[0].shape
-    strides = block_outs[0].stride()
-    for bo, bl in zip(block_outs, block_lses):
-        if bo.shape != (B, Sq, Hq, D) or bo.dtype != torch.bfloat16 or bo.stride() != strides or strides[-1] != 1:
-            raise RuntimeError("block outputs must be bfloat16 (B,Sq,Hq,D) with one set of strides")
-        if bl.shape != (B, Hq, Sq) or bl.dtype != torch.float32 or not bl.is_contiguous():
-            raise RuntimeError("block lse must be contiguous float32 (B,Hq,Sq)")
-    if final_out.shape != (B, Sq, Hq, D) or final_out.dtype != torch.bfloat16 or not final_out.is_contiguous():
+    B, Sq, Hq, D = final_out.shape
+    if final_out.dtype != torch.bfloat16 or not final_out.is_contiguous():
         raise RuntimeError("final_out must be contiguous bfloat16 (B,Sq,Hq,D)")
     if final_lse.shape != (B, Hq, Sq) or final_lse.dtype != torch.float32 or not final_lse.is_contiguous():
         raise RuntimeError("final_lse must be contiguous float32 (B,Hq,Sq)")
+    ss, sh = block_outs[0].stride(1), block_outs[0].stride(2)
+    for bo, bl, sb in zip(block_outs, block_lses, begins):
+        if not 0 <= sb <= Sq:
+            raise RuntimeError("row_begin outside the sequence")
+        if bo.shape != (B, Sq - sb, Hq, D) or bo.dtype != torch.bfloat16:
+            raise RuntimeError("block outputs must be bfloat16 (B, Sq - row_begin, Hq, D)")
+        if bo.stride(3) != 1 or (bo.stride(1), bo.stride(2)) != (ss, sh):
+            raise RuntimeError("block outputs need a contiguous head dimension and common row / head strides")
+        if bl.shape != (B, Hq, Sq - sb) or bl.dtype != torch.float32 or not bl.is_contiguous():
+            raise RuntimeError("block lse must be contiguous float32 (B, Hq, Sq - row_begin)")
     outs = (ctypes.c_void_p * n)(*[t.data_ptr() for t in block_outs])
     lses = (ctypes.c_void_p * n)(*[t.data_ptr() for t in block_lses])
+    sbs = (ctypes.c_int64 * n)(*[t.stride(0) for t in block_outs])
+    rbs = (ctypes.c_int * n)(*begins)
     with torch.cuda.device(final_out.device):
-        code = N.lib().mhip_lse_merge_many(outs, lses, n, N.ptr(final_out), N.ptr(final_lse), B, Sq, Hq, D,
-                                           strides[0], strides[1], strides[2], N.stream_of(final_out))
+        code = N.lib().mhip_lse_merge_many(outs, lses, sbs, rbs, n, N.ptr(final_out), N.ptr(final_lse),
+                                           B, Sq, Hq, D, ss, sh, N.stream_of(final_out))
     N.check(code, "mhip_lse_merge_many")
 
 

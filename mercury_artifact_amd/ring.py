@@ -221,7 +221,7 @@ def flash_attn_expose_reduce_q_ring(qs, kvs, os_, lses, softmax_scale, dropout_p
 
 
 def zigzag_causal_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=True, window_size=(-1, -1),
-                          alibi_slopes=None, deterministic=False, *, ring: LocalRing):
+                          alibi_slopes=None, deterministic=False, *, ring: LocalRing, deferred_merge: bool = True):
     """Causal forward step in the zigzag layout (rank r holds sequence blocks r and 2W-1-r).  Not in
     the reference, which only carries the ``slice_`` hook (utils/flash_attn_dsl.py:56,63-68); the
     three step classes are the diagonal (causal block), "first half of the chunk" and "second half
@@ -234,6 +234,9 @@ def zigzag_causal_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=True
         raise ValueError("zigzag needs an even number of local rows and equal Q / KV shards")
     half = Sq // 2
     _out = _lse = _kv = _next_kv = None
+    defer = (deferred_merge and world <= MAX_MERGE_MANY and o.dtype == torch.bfloat16
+             and o.is_contiguous() and lse.is_contiguous())
+    blocks = []
     for step in range(world):
         if step == 0:
             _kv = kv.contiguous()
@@ -254,7 +257,13 @@ def zigzag_causal_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=True
         outputs = _flash_attn_forward(**_fwd_params(bq, bk, bv, softmax_scale, dropout_p, bc,
                                                     window_size, alibi_slopes))
         block_out, block_lse, _, _ = outputs
+        if defer:
+            blocks.append((block_out, block_lse, 0 if sl is None else half))
+            continue
         _out, _lse = update_out_and_lse(_out, _lse, block_out, block_lse, slice_=sl)
+    if defer:
+        merge_many([b[0] for b in blocks], [b[1] for b in blocks], o, lse, row_begin=[b[2] for b in blocks])
+        return
     o[:, :, :, :] = _out.to(o.dtype)
     lse[:, :, :] = _lse.squeeze(dim=-1).transpose(1, 2)
 

@@ -73,17 +73,21 @@ def test_elementwise_rejects(lib):
     assert lib.mhip_flash_reduce(P, P + 4, P, 8, 128, None) == EALIGN
     assert lib.mhip_flash_reduce(P, P, P, -1, 128, None) == EINVAL
     assert lib.mhip_flash_reduce(P, P, P, 0, 128, None) == OK
-    import ctypes
     two = (ctypes.c_void_p * 2)(P, P)
-    many = lambda outs=two, lses=two, n=2, fo=P, fl=P, D=128, st=(128 * 4 * 8, 128 * 4, 128): \
-        lib.mhip_lse_merge_many(outs, lses, n, fo, fl, 1, 8, 4, D, *st, None)
+    sb2 = (ctypes.c_int64 * 2)(8 * 4 * 128, 8 * 4 * 128)
+
+    def many(outs=two, lses=two, sb=sb2, begin=None, n=2, fo=P, fl=P, D=128, st=(128 * 4, 128), B=1):
+        return lib.mhip_lse_merge_many(outs, lses, sb, begin, n, fo, fl, B, 8, 4, D, *st, None)
+
     assert many(n=0) == EINVAL and many(n=17) == EINVAL
-    assert many(fo=None) == EINVAL and many(outs=None) == EINVAL
+    assert many(fo=None) == EINVAL and many(outs=None) == EINVAL and many(sb=None) == EINVAL
     assert many(outs=(ctypes.c_void_p * 2)(P, None)) == EINVAL
+    assert many(begin=(ctypes.c_int * 2)(0, 9)) == EINVAL and many(begin=(ctypes.c_int * 2)(-1, 0)) == EINVAL
     assert many(outs=(ctypes.c_void_p * 2)(P, P + 8)) == EALIGN
-    assert many(st=(128 * 4 * 8, 128 * 4 + 4, 128)) == EALIGN
+    assert many(st=(128 * 4 + 4, 128)) == EALIGN
+    assert many(sb=(ctypes.c_int64 * 2)(4096, 4100)) == EALIGN
     assert many(D=40) == EUNSUPPORTED
-    assert lib.mhip_lse_merge_many(two, two, 2, P, P, 0, 8, 4, 128, 4096, 512, 128, None) == OK
+    assert many(B=0) == OK
     assert lib.mhip_tree_merge(P, None, P, 8, 128, 0, None) == EINVAL
     assert lib.mhip_tree_merge(P + 8, P, P, 8, 128, 1, None) == EALIGN
     assert lib.mhip_tree_merge(P, P, P, 0, 128, 1, None) == OK

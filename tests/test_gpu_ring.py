@@ -113,8 +113,9 @@ def test_packed_reduce_ring():
     _compare(o, lse, ro, rl)
 
 
+@pytest.mark.parametrize("deferred", [False, True])
 @pytest.mark.parametrize("rank", [0, 1, 3])
-def test_zigzag_causal_ring(rank):
+def test_zigzag_causal_ring(rank, deferred):
     """Causal GQA in the zigzag layout, a scaled-down Llama-3-8B shape (B2, Hq/Hkv = 4, D128)."""
     import mercury_artifact_amd as M
 
@@ -131,7 +132,8 @@ def test_zigzag_causal_ring(rank):
     qd = q[:, pos[rank]].cuda()
     o = torch.empty_like(qd)
     lse = torch.empty(B, Hq, 2 * block, dtype=torch.float32, device="cuda")
-    M.zigzag_causal_pack_kv(qd, dev[rank], o, lse, scale, ring=M.LocalRing((W,), rank, dev))
+    M.zigzag_causal_pack_kv(qd, dev[rank], o, lse, scale, ring=M.LocalRing((W,), rank, dev),
+                            deferred_merge=deferred)
     _compare(o, lse, ref_o[:, pos[rank]], ref_l[:, :, pos[rank]])
 
 
