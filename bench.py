@@ -26,6 +26,7 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # by its reading for the calibration launch at the end of main() (profiles/ring_step_config1_hbm_traffic.md)
 TRAFFIC_FWD_BYTES = 134.9e6
 TRAFFIC_MERGE_BYTES = 171.5e6
+TRAFFIC_MANY_BYTES = 321.0e6
 
 
 def cpu_baseline(sample_heads: int, B: int, Sq: int, D: int, W: int):
@@ -288,7 +289,7 @@ def main() -> int:
                      "traffic": TRAFFIC_FWD_BYTES, "avg_launch_ms": round(fwd_ms, 4), "launches": len(fwd_events)},
         "roofline_merge_many": {"bound": "hbm", "kernel": "lse_merge_many_kernel", "achieved": round(many_gbs, 1),
                                 "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(many_gbs / PEAK_HBM_GBS, 4),
-                                "traffic": None, "avg_launch_ms": round(many_ms, 5), "launches": len(many_events),
+                                "traffic": TRAFFIC_MANY_BYTES, "avg_launch_ms": round(many_ms, 5), "launches": len(many_events),
                                 "bytes_per_launch": many_bytes},
         "roofline_merge": {"bound": "hbm", "kernel": "lse_merge_kernel", "achieved": round(merge_gbs, 1),
                            "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(merge_gbs / PEAK_HBM_GBS, 4),
