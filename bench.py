@@ -82,6 +82,12 @@ def other_kernels(torch, M, dev):
     out["bwd_bf16_4096x4096"] = {"ms": round(ms, 4), "tflops": round(5 * unit / ms / 1e9, 1),
                                  "tflops_executed": round(7 * unit / ms / 1e9, 1),
                                  "flops": "10 B H Sq Sc D algorithmic; the two-pass kernel executes 14"}
+    # one rank's backward step over the same 8 chunks (dq accumulated in fp32 over the chunks, dk/dv per chunk)
+    chunks_b = [kv for _ in range(8)]                       # timing only: every chunk has the same bytes
+    ms = timeit(lambda: M.flash_attn_backward(q, kv, o, lse, do, dq, dkv, scale, ring=M.LocalRing((8,), 0, chunks_b)),
+                n=3, w=1)
+    out["step_bf16_backward_ring_4096x8"] = {"ms": round(ms, 3), "tflops": round(8 * 5 * unit / ms / 1e9, 1),
+                                             "flops": "8 chunks x 10 B H Sq Sc D algorithmic"}
     del dq, dkv, do
     S8 = 16384
     q8, sq = M.quantize_e4m3(torch.randn(B, S8, H, D, device=dev))

@@ -23,7 +23,7 @@ from typing import Optional
 
 import torch
 
-from .flash_attn_interface import _flash_attn_backward, _flash_attn_forward
+from .flash_attn_interface import _flash_attn_backward, _flash_attn_forward, attn_bwd_block
 from .merge import (MAX_MERGE_MANY, get_default_args, grad_accumulate, merge_into, merge_many, pack_block,
                     update_out_and_lse)
 from .schedule import (LocalRing, n_dim_to_one_dim, one_dim_to_n_dim, reduce_buffer_route, shift_tuple_element,
@@ -287,14 +287,21 @@ def fp8_pack_split_kv(q, kv, o, lse, softmax_scale, q_descale, k_descale, v_desc
 
 def flash_attn_backward(q, kv, o, lse, dout, dq, dkv, softmax_scale, dropout_p=0, causal=False,
                         window_size=(-1, -1), alibi_slopes=None, deterministic=False, *,
-                        ring: LocalRing, dkv_chunks: Optional[dict] = None):
+                        ring: LocalRing, dkv_chunks: Optional[dict] = None, fused_accumulate: bool = True):
     """Backward ring step (template utils/attn_bwd_dsl.py:37-135 after ``shift`` on the KV axis):
     KV chunks arrive in ring order, each gets a block backward against the local q / o / lse / dout;
     dq accumulates in fp32 over the chunks (utils/attn_bwd_dsl.py:117-122) and is stored as
     ``dq.dtype`` at the end (131-132).  The fp32 dK/dV accumulator that travels with its chunk on a
     real ring has exactly one contribution per rank, so here each chunk's block gradient is kept in
-    ``dkv_chunks[chunk id]`` (fp32) and the rank's own chunk is stored to ``dkv``."""
-    reduce_dq = None
+    ``dkv_chunks[chunk id]`` (fp32) and the rank's own chunk is stored to ``dkv``.
+
+    ``fused_accumulate=True`` (default) lets the block kernel add its fp32 dq straight into the accumulator
+    (one pass fewer over it per chunk, and the sum sees the unrounded block gradient) and casts a chunk's
+    dK/dV to fp32 only when ``dkv_chunks`` asks for it; ``False`` is the literal sequence: block backward
+    through ``_flash_attn_backward(**params)``, then ``torch.add`` on the bf16 block gradients."""
+    if dropout_p != 0 or alibi_slopes is not None or tuple(window_size) != (-1, -1):
+        fused_accumulate = False                # let the operator report what it does not support
+    reduce_dq = torch.zeros(q.shape, dtype=torch.float32, device=q.device) if fused_accumulate else None
     _kv = _next_kv = None
     own = ring.current
     for step, hop in enumerate(_hops(ring)):
@@ -310,6 +317,14 @@ def flash_attn_backward(q, kv, o, lse, dout, dq, dkv, softmax_scale, dropout_p=0
             ring.commit()
         block_dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
         block_dkv = torch.empty(_kv.shape, dtype=kv.dtype, device=kv.device)
+        if fused_accumulate:
+            attn_bwd_block(dout, q, _kv[0], _kv[1], o, lse, block_dq, block_dkv[0], block_dkv[1], softmax_scale,
+                           causal=False, deterministic=deterministic, dq_acc=reduce_dq)
+            if dkv_chunks is not None:
+                dkv_chunks[chunk_id] = grad_accumulate(None, block_dkv)
+            if chunk_id == own:
+                dkv[...] = block_dkv
+            continue
         params = get_default_args(_flash_attn_backward).copy()
         params.update({
             "dout": dout, "q": q, "k": _kv[0], "v": _kv[1], "out": o, "softmax_lse": lse,

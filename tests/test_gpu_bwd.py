@@ -104,7 +104,8 @@ def test_bwd_dq_accumulator_and_determinism():
     assert _rel(acc.cpu(), 2 * rdq) <= 5e-3             # fp32 accumulation of two identical blocks
 
 
-def test_bwd_ring_step():
+@pytest.mark.parametrize("fused", [False, True])
+def test_bwd_ring_step(fused):
     """The backward ring step (utils/attn_bwd_dsl.py:70-134 after `shift`): dq accumulates over the chunks,
     each chunk's dk/dv is compared with the oracle's."""
     import mercury_artifact_amd as M
@@ -124,7 +125,7 @@ def test_bwd_ring_step():
     dkv = torch.empty_like(dev[rank])
     got = {}
     M.flash_attn_backward(q.cuda(), dev[rank], o16.cuda(), lse.cuda(), dout.cuda(), dq, dkv, scale,
-                          ring=M.LocalRing((W,), rank, dev), dkv_chunks=got)
+                          ring=M.LocalRing((W,), rank, dev), dkv_chunks=got, fused_accumulate=fused)
     torch.cuda.synchronize()
     _check_grad("dq", dq, rdq)
     assert sorted(got) == list(range(W))
