@@ -268,6 +268,21 @@ def main() -> int:
     torch.cuda.synchronize()
     del calib
 
+    # what a plain device-to-device copy of 256 MiB reaches on this box (read + write bytes over time): the
+    # practical ceiling next to the 8 TB/s the merge kernels are priced against
+    src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev).normal_()
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    c0.record()
+    for _ in range(10):
+        dst.copy_(src)
+    c1.record()
+    torch.cuda.synchronize()
+    copy_gbs = 2 * src.numel() * 4 / (c0.elapsed_time(c1) / 10 * 1e-3) / 1e9
+    del src, dst
+
     variants = None if args.no_variants else other_kernels(torch, M, dev)
 
     props = torch.cuda.get_device_properties(0)
@@ -289,7 +304,8 @@ def main() -> int:
                    "flops_per_step": flops_per_step, "pct_of_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
                    "literal_merge_chain_ms_per_step": round(unfused_ms, 4),
                    "hip_graph_ms_per_step": graph_ms, "hip_graph_bit_identical": graph_same,
-                   "device": props.gcnArchName, "cus": props.multi_processor_count},
+                   "device": props.gcnArchName, "cus": props.multi_processor_count,
+                   "d2d_copy_gbs": round(copy_gbs, 1)},
         "roofline": {"bound": "mfma", "kernel": "attn_fwd_bf16_d128", "achieved": round(fwd_tflops, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(fwd_tflops / PEAK_BF16_TFLOPS, 4),
                      "traffic": TRAFFIC_FWD_BYTES, "avg_launch_ms": round(fwd_ms, 4), "launches": len(fwd_events)},
