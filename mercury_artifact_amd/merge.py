@@ -120,6 +120,14 @@ def merge_many(block_outs: Sequence[torch.Tensor], block_lses: Sequence[torch.Te
             raise RuntimeError("block outputs need a contiguous head dimension and common row / head strides")
         if bl.shape != (B, Hq, Sq - sb) or bl.dtype != torch.float32 or not bl.is_contiguous():
             raise RuntimeError("block lse must be contiguous float32 (B, Hq, Sq - row_begin)")
+    if B * Sq * Hq == 0:
+        return
+    # a block that starts past the last row contributes nothing (and has no memory to point at)
+    keep = [i for i in range(n) if begins[i] < Sq]
+    if not keep:
+        raise RuntimeError("merge_many needs at least one block that covers a row")
+    block_outs, block_lses = [block_outs[i] for i in keep], [block_lses[i] for i in keep]
+    begins, n = [begins[i] for i in keep], len(keep)
     outs = (ctypes.c_void_p * n)(*[t.data_ptr() for t in block_outs])
     lses = (ctypes.c_void_p * n)(*[t.data_ptr() for t in block_lses])
     sbs = (ctypes.c_int64 * n)(*[t.stride(0) for t in block_outs])

@@ -244,14 +244,15 @@ def test_merge_many_with_partial_row_ranges():
     import mercury_artifact_amd as M
 
     B, Sq, H, D = 2, 40, 3, 128
-    begins = [0, 20, 0, 20, 33]
+    begins = [0, 20, 0, 20, 33, 40]                    # the last block starts past the end: no rows
     g = torch.Generator().manual_seed(9)
     outs = [torch.randn(B, Sq - sb, H, D, generator=g).bfloat16() for sb in begins]
     lses = [torch.randn(B, H, Sq - sb, generator=g) * 2 + 1 for sb in begins]
     out = lse = None
     for bo, bl, sb in zip(outs, lses, begins):
         sl = None if sb == 0 else (slice(None), slice(sb, None))
-        out, lse = O.update_out_and_lse(out, lse, bo, bl, slice_=sl, acc_dtype=torch.float64)
+        if sb < Sq:
+            out, lse = O.update_out_and_lse(out, lse, bo, bl, slice_=sl, acc_dtype=torch.float64)
     ro, rl = out.float(), lse.squeeze(-1).transpose(1, 2).float()
     fo = torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device="cuda")
     fl = torch.empty(B, H, Sq, dtype=torch.float32, device="cuda")
@@ -259,4 +260,4 @@ def test_merge_many_with_partial_row_ranges():
     assert ((fo.float().cpu() - ro).abs() - (1e-3 + 2 ** -8 * ro.abs())).max().item() <= 0
     assert torch.allclose(fl.cpu(), rl, atol=1e-5, rtol=1e-5)
     with pytest.raises(RuntimeError):
-        M.merge_many([t.cuda() for t in outs], [t.cuda() for t in lses], fo, fl, row_begin=[0] * 5)
+        M.merge_many([t.cuda() for t in outs], [t.cuda() for t in lses], fo, fl, row_begin=[0] * 6)

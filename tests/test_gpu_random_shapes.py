@@ -1,4 +1,4 @@
-"""Seeded random small shapes through the three block kernels against the CPU oracle: ragged row and key
+"""Seeded random small shapes through the three block kernels and the one-pass fold against the CPU oracle: ragged row and key
 counts, batch 1-3, 1-4 query heads per KV head, with and without the causal mask.  Tolerances as in the
 per-kernel test files."""
 import random
@@ -94,3 +94,35 @@ def test_random_fp8_forward(B, Sq, Sc, Hq, Hkv, causal):
     fin = ~torch.isinf(la)
     if fin.any():
         assert ((lse[fin] - la[fin]).abs() / la[fin].abs().clamp_min(1.0)).max().item() <= 1e-3
+
+
+def _fold_cases(seed, n):
+    rng = random.Random(seed)
+    return [(rng.randint(1, 3), rng.randint(1, 300), rng.randint(1, 6), rng.choice([64, 128, 256]), rng.randint(1, 16))
+            for _ in range(n)]
+
+
+@pytest.mark.parametrize("B,Sq,H,D,n", _fold_cases(404, 12))
+def test_random_fold_of_block_results(B, Sq, H, D, n):
+    """merge_many on random shapes and block counts, some blocks covering only a tail of the rows, against the
+    chain of reference merges in fp64 (bf16 result: atol 1e-3 + rtol 2^-8; lse 1e-5)."""
+    import mercury_artifact_amd as M
+
+    print(f"fold B{B} Sq{Sq} H{H} D{D} n{n}", flush=True)
+    rng = random.Random(B * 7919 + Sq * 31 + n)
+    g = torch.Generator().manual_seed(B * 1000003 + Sq * 1009 + n)
+    begins = [0] + [rng.choice([0, 0, rng.randint(0, Sq)]) for _ in range(n - 1)]
+    outs = [torch.randn(B, Sq - sb, H, D, generator=g).bfloat16() for sb in begins]
+    lses = [torch.randn(B, H, Sq - sb, generator=g) * 4 for sb in begins]
+    out = lse = None
+    for bo, bl, sb in zip(outs, lses, begins):
+        if bo.shape[1] == 0:
+            continue
+        sl = None if sb == 0 else (slice(None), slice(sb, None))
+        out, lse = O.update_out_and_lse(out, lse, bo, bl, slice_=sl, acc_dtype=torch.float64)
+    ro, rl = out.float(), lse.squeeze(-1).transpose(1, 2).float()
+    fo = torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device="cuda")
+    fl = torch.empty(B, H, Sq, dtype=torch.float32, device="cuda")
+    M.merge_many([t.cuda() for t in outs], [t.cuda() for t in lses], fo, fl, row_begin=begins)
+    assert ((fo.float().cpu() - ro).abs() - (1e-3 + 2 ** -8 * ro.abs())).max().item() <= 0
+    assert ((fl.cpu() - rl).abs() / rl.abs().clamp_min(1.0)).max().item() <= 1e-5
