@@ -35,6 +35,7 @@ def namespace() -> dict:
         "update_out_and_lse": update_out_and_lse,
         "_update_out_and_lse": _update_out_and_lse,
         "flash_reduce": flash_reduce,
+        "merge_many": merge_many,
         "update_out_and_lse_collective": update_out_and_lse_collective,
         "add_collective": add_collective,
         "one_dim_to_n_dim": one_dim_to_n_dim,
