@@ -93,6 +93,44 @@ def test_fwd_block_peaked_logits():
     _check(out, lse, ro, rl, "peaked")
 
 
+@pytest.mark.parametrize("direction", ["rising", "falling"])
+@pytest.mark.parametrize("fp8", [False, True])
+def test_fwd_block_monotone_scores(direction, fp8):
+    """Scores that rise (or fall) by about 20 binades from one key tile to the next: with rising scores the
+    reference the exponentials are taken against has to move on every tile and everything accumulated so far is
+    rescaled by 2^-20 each time; with falling scores it must never move and later tiles underflow to nothing.
+    The first 16 head-dim values carry the ramp, the rest is noise."""
+    import mercury_artifact_amd as M
+
+    B, Sq, Sc, H, D = 1, 96, 640, 2, 128
+    g = torch.Generator().manual_seed(7)
+    q = torch.randn(B, Sq, H, D, generator=g) * 0.25
+    k = torch.randn(B, Sc, H, D, generator=g) * 0.25
+    v = torch.randn(B, Sc, H, D, generator=g)
+    ramp = torch.arange(Sc, dtype=torch.float32) / 64.0              # one unit per 64-key tile
+    if direction == "falling":
+        ramp = ramp.flip(0)
+    q[..., :16] = 2.0
+    k[..., :16] = (ramp * 5.0)[None, :, None, None] / 2.0            # q.k ramp = 16 * 2 * 2.5 * t = 80 t
+    scale = D ** -0.5                                                # 80 * 0.088 * log2(e) = 10 binades per unit
+    k[..., :16] *= 2.0                                               # -> 20 binades per tile
+    if fp8:
+        (qq, sq), (kq, sk), (vq, sv) = M.quantize_e4m3(q.cuda()), M.quantize_e4m3(k.cuda()), M.quantize_e4m3(v.cuda())
+        ref_q, ref_k, ref_v = (O.dequantize(t.cpu(), s_.cpu()) for t, s_ in ((qq, sq), (kq, sk), (vq, sv)))
+        ro, rl = O.block_attention(ref_q, ref_k, ref_v, scale)
+        out, lse = M.attn_fwd_block(qq, kq, vq, scale, q_descale=sq, k_descale=sk, v_descale=sv)
+        tol = 6e-2
+    else:
+        qb, kb, vb = q.bfloat16(), k.bfloat16(), v.bfloat16()
+        ro, rl = O.block_attention(qb.float(), kb.float(), vb.float(), scale)
+        out, lse = M.attn_fwd_block(qb.cuda(), kb.cuda(), vb.cuda(), scale)
+        tol = 2e-2
+    out, lse = out.float().cpu(), lse.cpu()
+    assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+    assert (out - ro).abs().max().item() <= tol
+    assert ((lse - rl).abs() / rl.abs().clamp_min(1.0)).max().item() <= 1e-3
+
+
 def test_fwd_block_strided_views_and_guard_bands():
     """k / v as halves of one packed tensor (storage offset != 0 for v), q as a row slice of a larger
     tensor, out written into the middle of a sentinel-filled buffer."""
