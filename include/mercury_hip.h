@@ -149,7 +149,8 @@ int mhip_tree_merge(const float* src, const float* row_max, float* dst, int64_t 
  * Pack a block result: dst (B,Sq,Hq,D+1) fp32 contiguous =
  * cat([float(block_out), block_lse^T], -1)   (utils/flash_attn_dsl.py:396).
  * If lhs is not NULL the pack is fused with the reduce: dst = flash_reduce(lhs, pack(block));
- * dst must not overlap lhs.  block_out (B,Sq,Hq,D) bf16 and block_lse (B,Hq,Sq) contiguous.
+ * dst must not overlap lhs; dst and lhs 16-byte aligned.  block_out (B,Sq,Hq,D) bf16 and block_lse
+ * (B,Hq,Sq) contiguous.
  */
 int mhip_pack_reduce(const float* lhs, const void* block_out, const float* block_lse,
                      float* dst, int B, int Sq, int Hq, int D, void* stream);

@@ -267,148 +267,148 @@ void launch_merge8(const MergeParams& p, bool first, bool fin, hipStream_t st) {
 }
 
 // ---- packed form -----------------------------------------------------------------------------------
-// The buffers are flat fp32 arrays of rows x (D+1); a row is 4(D+1) bytes long, which is not a
-// multiple of 16 for D = 128, so the kernel walks the flat array in aligned groups of four floats
-// and looks up the row (and its two LSEs) of every element.  Threads read the LSE column of rows
-// whose other elements belong to other threads, so dst must not overlap lhs or rhs.
-__global__ __launch_bounds__(256) void flash_reduce_kernel(const float* __restrict__ lhs,
-                                                           const float* __restrict__ rhs,
-                                                           float* __restrict__ dst,
-                                                           int64_t total, int W) {
-  const int64_t g = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
-  if (g >= total) return;
-  float a[4], b[4];
-  if (g + 4 <= total) {
-    const f32x4 va = *reinterpret_cast<const f32x4*>(lhs + g);
-    const f32x4 vb = *reinterpret_cast<const f32x4*>(rhs + g);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) { a[j] = va[j]; b[j] = vb[j]; }
-  } else {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      a[j] = g + j < total ? lhs[g + j] : 0.f;
-      b[j] = g + j < total ? rhs[g + j] : 0.f;
-    }
-  }
-  const int64_t row_a = g / W;
-  float w0, n0, w1 = 0.f, n1 = 0.f;
-  merge_weights(lhs[row_a * W + W - 1], rhs[row_a * W + W - 1], w0, n0);
-  const int64_t row_b = (g + 3) / W;
-  if (row_b != row_a && row_b * W + W - 1 < total)
-    merge_weights(lhs[row_b * W + W - 1], rhs[row_b * W + W - 1], w1, n1);
-  float r[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int64_t e = g + j;
-    const bool second = e / W != row_a;
-    const float w = second ? w1 : w0;
-    const float nl = second ? n1 : n0;
-    r[j] = (e % W == W - 1) ? nl : a[j] - w * (a[j] - b[j]);
-  }
-  if (g + 4 <= total) {
-    f32x4 v = {r[0], r[1], r[2], r[3]};
-    *reinterpret_cast<f32x4*>(dst + g) = v;
-  } else {
-    for (int j = 0; j < 4 && g + j < total; ++j) dst[g + j] = r[j];
-  }
-}
-
-// Tree-attention merge of packed (rows x W) = (out | lse) operands across ranks
-// (utils/flash_attn_dsl.py:307-324): with m = max over ranks of lse,
+// flash_reduce (utils/flash_attn_dsl.py:293-305), the pack that feeds it (utils/flash_attn_dsl.py:396) and
+// the tree-attention merge (utils/flash_attn_dsl.py:307-324) work on flat fp32 arrays of rows x (D+1),
+// the LSE in the last column.  A row is 4(D+1) bytes long, which is not a multiple of 16 for D = 128, so
+// the kernels walk the flat array in aligned groups of four floats: one division per thread (by a
+// compile-time row width when D = 128) places the group, and its four elements sit in at most two rows,
+// found by stepping.  Threads read the LSE column of rows whose other elements belong to other threads,
+// so dst must not overlap the inputs.  IT is the index type: 32 bits for buffers of fewer than 2^31
+// elements, 64 bits otherwise.
+//
+// Tree-attention merge: with m = max over ranks of lse,
 //   prepare: dst = (out * d | d),  d = exp(lse - m)      -- what every rank contributes to the SUM
 //   finish:  dst = (sum_out / sum_d | m + log(sum_d))    -- from the summed contributions
 // Packing d next to out * d makes the SUM one collective instead of the reference's two.  Rows whose
-// lse is -inf everywhere (m = -inf) contribute d = 0 and finish as (0 | -inf).  Same flat walk in aligned
-// groups of four floats as flash_reduce_kernel; `aux` is the per-row maximum, contiguous.
-template <bool FINISH>
-__global__ __launch_bounds__(256) void tree_merge_kernel(const float* __restrict__ src,
-                                                         const float* __restrict__ aux,
-                                                         float* __restrict__ dst, int64_t total, int W) {
-  const int64_t g = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+// lse is -inf everywhere (m = -inf) contribute d = 0 and finish as (0 | -inf).  `aux` is the per-row
+// maximum, contiguous.
+template <typename IT>
+struct PackedPos {
+  IT row;                 // of the group's first element
+  uint32_t col;
+};
+template <int WCT, typename IT>
+__device__ __forceinline__ PackedPos<IT> packed_pos(IT g, uint32_t w_rt) {
+  const uint32_t W = WCT ? (uint32_t)WCT : w_rt;
+  PackedPos<IT> p;
+  p.row = g / W;
+  p.col = (uint32_t)(g - p.row * W);
+  return p;
+}
+template <typename IT>
+__device__ __forceinline__ f32x4 load4(const float* base, IT g, IT total) {
+  if (g + 4 <= total) return *reinterpret_cast<const f32x4*>(base + g);
+  f32x4 v = {0.f, 0.f, 0.f, 0.f};
+  for (IT j = 0; j < 4 && g + j < total; ++j) v[j] = base[g + j];
+  return v;
+}
+template <typename IT>
+__device__ __forceinline__ void store4(float* base, IT g, IT total, const f32x4& v) {
+  if (g + 4 <= total) { *reinterpret_cast<f32x4*>(base + g) = v; return; }
+  for (IT j = 0; j < 4 && g + j < total; ++j) base[g + j] = v[j];
+}
+
+template <int WCT, typename IT>
+__global__ __launch_bounds__(256) void flash_reduce_kernel(const float* __restrict__ lhs, const float* __restrict__ rhs,
+                                                           float* __restrict__ dst, IT total, uint32_t w_rt) {
+  const uint32_t W = WCT ? (uint32_t)WCT : w_rt;
+  const IT g = ((IT)blockIdx.x * 256u + threadIdx.x) * 4u;
   if (g >= total) return;
-  float a[4];
-  if (g + 4 <= total) {
-    const f32x4 va = *reinterpret_cast<const f32x4*>(src + g);
+  const PackedPos<IT> pos = packed_pos<WCT, IT>(g, w_rt);
+  const f32x4 a = load4<IT>(lhs, g, total), b = load4<IT>(rhs, g, total);
+  float w[2] = {0.f, 0.f}, nl[2] = {0.f, 0.f};
+  const IT last0 = pos.row * W + W - 1;
+  merge_weights(lhs[last0], rhs[last0], w[0], nl[0]);
+  if (pos.col + 3 >= W && last0 + W < total) merge_weights(lhs[last0 + W], rhs[last0 + W], w[1], nl[1]);
+  f32x4 r;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) a[j] = va[j];
-  } else {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) a[j] = g + j < total ? src[g + j] : 0.f;
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t c = pos.col + j;
+    const int k = c >= W ? 1 : 0;
+    const uint32_t cc = k ? c - W : c;
+    r[j] = cc == W - 1 ? nl[k] : a[j] - w[k] * (a[j] - b[j]);
   }
-  const int64_t row_a = g / W;
-  const int64_t row_b = (g + 3) / W;
-  // per-row factor and last-column value, for the (at most) two rows this group touches
+  store4<IT>(dst, g, total, r);
+}
+
+template <bool FINISH, int WCT, typename IT>
+__global__ __launch_bounds__(256) void tree_merge_kernel(const float* __restrict__ src, const float* __restrict__ aux,
+                                                         float* __restrict__ dst, IT total, uint32_t w_rt) {
+  const uint32_t W = WCT ? (uint32_t)WCT : w_rt;
+  const IT g = ((IT)blockIdx.x * 256u + threadIdx.x) * 4u;
+  if (g >= total) return;
+  const PackedPos<IT> pos = packed_pos<WCT, IT>(g, w_rt);
+  const f32x4 a = load4<IT>(src, g, total);
   float f[2] = {0.f, 0.f}, last[2] = {0.f, 0.f};
 #pragma unroll
   for (int k = 0; k < 2; ++k) {
-    const int64_t row = k == 0 ? row_a : row_b;
-    if (k == 1 && (row_b == row_a || row_b * W + W - 1 >= total)) break;
+    const IT row = pos.row + k;
+    if (k == 1 && !(pos.col + 3 >= W && row * W + W - 1 < total)) break;
     const float m = aux[row];
     const float tail = src[row * W + W - 1];
     if (!FINISH) {
-      const float d = (m == -INFINITY) ? 0.f : __expf(tail - m);      // tail = this rank's lse
+      const float d = (m == -INFINITY) ? 0.f : __expf(tail - m);
       f[k] = d;
       last[k] = d;
     } else {
-      f[k] = tail > 0.f ? 1.f / tail : 0.f;                           // tail = summed d
+      f[k] = tail > 0.f ? 1.f / tail : 0.f;
       last[k] = tail > 0.f ? m + __logf(tail) : -INFINITY;
     }
   }
-  float r[4];
+  f32x4 r;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int64_t e = g + j;
-    const int k = (e / W != row_a) ? 1 : 0;
-    r[j] = (e % W == W - 1) ? last[k] : a[j] * f[k];
+    const uint32_t c = pos.col + j;
+    const int k = c >= W ? 1 : 0;
+    const uint32_t cc = k ? c - W : c;
+    r[j] = cc == W - 1 ? last[k] : a[j] * f[k];
   }
-  if (g + 4 <= total) {
-    f32x4 v = {r[0], r[1], r[2], r[3]};
-    *reinterpret_cast<f32x4*>(dst + g) = v;
-  } else {
-    for (int j = 0; j < 4 && g + j < total; ++j) dst[g + j] = r[j];
-  }
+  store4<IT>(dst, g, total, r);
 }
 
-// dst (rows x (D+1)) = pack(block)  or  flash_reduce(lhs, pack(block)); same flat walk over dst.
-template <bool REDUCE>
+template <bool REDUCE, int WCT, typename IT>
 __global__ __launch_bounds__(256) void pack_reduce_kernel(const float* __restrict__ lhs,
                                                           const uint16_t* __restrict__ block_out,
                                                           const float* __restrict__ block_lse,
-                                                          float* __restrict__ dst,
-                                                          int64_t total, int D, int Sq, int Hq) {
-  const int W = D + 1;
-  const int64_t g = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+                                                          float* __restrict__ dst, IT total, uint32_t w_rt,
+                                                          uint32_t Sq, uint32_t Hq) {
+  const uint32_t W = WCT ? (uint32_t)WCT : w_rt, D = W - 1;
+  const IT g = ((IT)blockIdx.x * 256u + threadIdx.x) * 4u;
   if (g >= total) return;
-  float r[4];
+  const PackedPos<IT> pos = packed_pos<WCT, IT>(g, w_rt);
+  uint32_t h = (uint32_t)(pos.row % Hq);
+  const IT bs = pos.row / Hq;
+  uint32_t s = (uint32_t)(bs % Sq);
+  IT b = bs / Sq;
+  f32x4 a = {0.f, 0.f, 0.f, 0.f};
+  if (REDUCE) a = load4<IT>(lhs, g, total);
+  float w[2] = {1.f, 1.f}, nl[2] = {0.f, 0.f};
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const IT row = pos.row + k;
+    if (k == 1) {
+      if (!(pos.col + 3 >= W && row * W < total)) break;
+      if (++h == Hq) { h = 0; if (++s == Sq) { s = 0; ++b; } }
+    }
+    const float bl = block_lse[(b * Hq + h) * Sq + s];
+    nl[k] = bl;
+    if (REDUCE) merge_weights(lhs[row * W + D], bl, w[k], nl[k]);
+  }
+  f32x4 r;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int64_t e = g + j;
-    if (e >= total) { r[j] = 0.f; continue; }
-    const int64_t row = e / W;
-    const int col = (int)(e % W);
-    const int h = (int)(row % Hq);
-    const int64_t bs = row / Hq;
-    const int s = (int)(bs % Sq);
-    const int64_t b = bs / Sq;
-    const float bl = block_lse[(b * Hq + h) * Sq + s];
-    float w = 1.f, nl = bl, a = 0.f;
-    if (REDUCE) {
-      merge_weights(lhs[row * W + D], bl, w, nl);
-      a = lhs[e];
-    }
-    if (col == D) {
-      r[j] = nl;
+    const uint32_t c = pos.col + j;
+    const int k = c >= W ? 1 : 0;
+    const uint32_t cc = k ? c - W : c;
+    if (g + j >= total) { r[j] = 0.f; continue; }
+    if (cc == D) {
+      r[j] = nl[k];
     } else {
-      const float bo = bf16_lo(block_out[row * D + col]);
-      r[j] = REDUCE ? a - w * (a - bo) : bo;
+      const float bo = bf16_lo(block_out[(pos.row + k) * D + cc]);
+      r[j] = REDUCE ? a[j] - w[k] * (a[j] - bo) : bo;
     }
   }
-  if (g + 4 <= total) {
-    f32x4 v = {r[0], r[1], r[2], r[3]};
-    *reinterpret_cast<f32x4*>(dst + g) = v;
-  } else {
-    for (int j = 0; j < 4 && g + j < total; ++j) dst[g + j] = r[j];
-  }
+  store4<IT>(dst, g, total, r);
 }
 
 // ---- all blocks of a step at once --------------------------------------------------------------------
@@ -630,8 +630,15 @@ extern "C" int mhip_flash_reduce(const float* lhs, const float* rhs, float* dst,
   if (!aligned16(lhs) || !aligned16(rhs) || !aligned16(dst)) return MHIP_EALIGN;
   const int64_t total = rows * (D + 1);
   const int64_t groups = (total + 3) / 4;
-  hipLaunchKernelGGL(flash_reduce_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), lhs, rhs, dst, total, D + 1);
+  const dim3 grid((unsigned)((groups + 255) / 256)), block(256);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const uint32_t w = (uint32_t)(D + 1);
+  if (total < (int64_t(1) << 31)) {
+    if (D == 128) hipLaunchKernelGGL((flash_reduce_kernel<129, uint32_t>), grid, block, 0, st, lhs, rhs, dst, (uint32_t)total, w);
+    else hipLaunchKernelGGL((flash_reduce_kernel<0, uint32_t>), grid, block, 0, st, lhs, rhs, dst, (uint32_t)total, w);
+  } else {
+    hipLaunchKernelGGL((flash_reduce_kernel<0, uint64_t>), grid, block, 0, st, lhs, rhs, dst, (uint64_t)total, w);
+  }
   return launch_status();
 }
 
@@ -645,8 +652,18 @@ extern "C" int mhip_tree_merge(const float* src, const float* row_max, float* ds
   const int64_t groups = (total + 3) / 4;
   const dim3 grid((unsigned)((groups + 255) / 256)), block(256);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (finish) hipLaunchKernelGGL(tree_merge_kernel<true>, grid, block, 0, st, src, row_max, dst, total, D + 1);
-  else hipLaunchKernelGGL(tree_merge_kernel<false>, grid, block, 0, st, src, row_max, dst, total, D + 1);
+  const uint32_t w = (uint32_t)(D + 1);
+  if (total < (int64_t(1) << 31)) {
+    const uint32_t t32 = (uint32_t)total;
+    if (finish && D == 128) hipLaunchKernelGGL((tree_merge_kernel<true, 129, uint32_t>), grid, block, 0, st, src, row_max, dst, t32, w);
+    else if (finish) hipLaunchKernelGGL((tree_merge_kernel<true, 0, uint32_t>), grid, block, 0, st, src, row_max, dst, t32, w);
+    else if (D == 128) hipLaunchKernelGGL((tree_merge_kernel<false, 129, uint32_t>), grid, block, 0, st, src, row_max, dst, t32, w);
+    else hipLaunchKernelGGL((tree_merge_kernel<false, 0, uint32_t>), grid, block, 0, st, src, row_max, dst, t32, w);
+  } else if (finish) {
+    hipLaunchKernelGGL((tree_merge_kernel<true, 0, uint64_t>), grid, block, 0, st, src, row_max, dst, (uint64_t)total, w);
+  } else {
+    hipLaunchKernelGGL((tree_merge_kernel<false, 0, uint64_t>), grid, block, 0, st, src, row_max, dst, (uint64_t)total, w);
+  }
   return launch_status();
 }
 
@@ -661,12 +678,20 @@ extern "C" int mhip_pack_reduce(const float* lhs, const void* block_out, const f
   const int64_t groups = (total + 3) / 4;
   const dim3 grid((unsigned)((groups + 255) / 256)), block(256);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (lhs)
-    hipLaunchKernelGGL(pack_reduce_kernel<true>, grid, block, 0, st, lhs,
-                       static_cast<const uint16_t*>(block_out), block_lse, dst, total, D, Sq, Hq);
-  else
-    hipLaunchKernelGGL(pack_reduce_kernel<false>, grid, block, 0, st, lhs,
-                       static_cast<const uint16_t*>(block_out), block_lse, dst, total, D, Sq, Hq);
+  const uint16_t* bo = static_cast<const uint16_t*>(block_out);
+  if (lhs && !aligned16(lhs)) return MHIP_EALIGN;
+  const uint32_t w = (uint32_t)(D + 1), sq = (uint32_t)Sq, hq = (uint32_t)Hq;
+  if (total < (int64_t(1) << 31)) {
+    const uint32_t t32 = (uint32_t)total;
+    if (lhs && D == 128) hipLaunchKernelGGL((pack_reduce_kernel<true, 129, uint32_t>), grid, block, 0, st, lhs, bo, block_lse, dst, t32, w, sq, hq);
+    else if (lhs) hipLaunchKernelGGL((pack_reduce_kernel<true, 0, uint32_t>), grid, block, 0, st, lhs, bo, block_lse, dst, t32, w, sq, hq);
+    else if (D == 128) hipLaunchKernelGGL((pack_reduce_kernel<false, 129, uint32_t>), grid, block, 0, st, lhs, bo, block_lse, dst, t32, w, sq, hq);
+    else hipLaunchKernelGGL((pack_reduce_kernel<false, 0, uint32_t>), grid, block, 0, st, lhs, bo, block_lse, dst, t32, w, sq, hq);
+  } else if (lhs) {
+    hipLaunchKernelGGL((pack_reduce_kernel<true, 0, uint64_t>), grid, block, 0, st, lhs, bo, block_lse, dst, (uint64_t)total, w, sq, hq);
+  } else {
+    hipLaunchKernelGGL((pack_reduce_kernel<false, 0, uint64_t>), grid, block, 0, st, lhs, bo, block_lse, dst, (uint64_t)total, w, sq, hq);
+  }
   return launch_status();
 }
 

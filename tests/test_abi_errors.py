@@ -92,6 +92,7 @@ def test_elementwise_rejects(lib):
     assert lib.mhip_tree_merge(P + 8, P, P, 8, 128, 1, None) == EALIGN
     assert lib.mhip_tree_merge(P, P, P, 0, 128, 1, None) == OK
     assert lib.mhip_pack_reduce(None, P, P, None, 1, 8, 2, 128, None) == EINVAL
+    assert lib.mhip_pack_reduce(P + 4, P, P, P, 1, 8, 2, 128, None) == EALIGN
     assert lib.mhip_pack_reduce(None, P, P, P, 0, 8, 2, 128, None) == OK
     assert lib.mhip_grad_accumulate(None, P, None, 16, None) == EINVAL
     assert lib.mhip_grad_accumulate(None, P + 2, P, 16, None) == EALIGN
