@@ -36,6 +36,7 @@ extern "C" {
 /* ---- element types -------------------------------------------------------------- */
 #define MHIP_BF16  0
 #define MHIP_E4M3  1   /* OCP float8 e4m3fn */
+#define MHIP_F32   2   /* input type of mhip_quantize_e4m3 only */
 
 /* ---- mask classes of one (Q shard, KV chunk) block -------------------------------- */
 #define MHIP_MASK_NONE    0
@@ -144,6 +145,17 @@ int mhip_flash_reduce(const float* lhs, const float* rhs, float* dst,
  * dst may alias src.  Rows with row_max = -inf come out as (0 | -inf). */
 int mhip_tree_merge(const float* src, const float* row_max, float* dst, int64_t rows, int D, int finish,
                     void* stream);
+
+/*
+ * Per-tensor e4m3 quantisation for the fp8 forward path (not in the reference, whose ring templates run
+ * bf16 only; the block kernel's descales are the scales this writes): scale = amax(|x|) / 448 (1 when the
+ * tensor is all zero), xq = round-to-nearest-even e4m3fn(clamp(x / scale, -448, 448)), bit for bit what
+ * (x.float() / scale).clamp(-448, 448).to(torch.float8_e4m3fn) gives.  x: n contiguous elements of
+ * MHIP_F32 or MHIP_BF16, 16-byte aligned; xq: n bytes, 8-byte aligned; scale: one fp32 on the device;
+ * amax_ws: 4 bytes of device scratch.  Three launches on the stream.
+ */
+int mhip_quantize_e4m3(const void* x, int dtype, int64_t n, void* xq, float* scale, float* amax_ws,
+                       void* stream);
 
 /*
  * Pack a block result: dst (B,Sq,Hq,D+1) fp32 contiguous =

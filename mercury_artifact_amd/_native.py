@@ -16,7 +16,7 @@ import torch
 LIB_PATH = os.environ.get("MERCURY_HIP_LIB") or os.path.join(
     os.path.dirname(os.path.abspath(__file__)), "csrc", "libmercury_hip.so")
 
-MHIP_BF16, MHIP_E4M3 = 0, 1
+MHIP_BF16, MHIP_E4M3, MHIP_F32 = 0, 1, 2
 MASK_NONE, MASK_CAUSAL = 0, 1
 
 _lib = None
@@ -34,6 +34,7 @@ _SIGNATURES = {
     "mhip_tree_merge": (c_int, [_P] * 3 + [_L, _I, _I, _P]),
     "mhip_pack_reduce": (c_int, [_P] * 4 + [_I] * 4 + [_P]),
     "mhip_grad_accumulate": (c_int, [_P] * 3 + [_L, _P]),
+    "mhip_quantize_e4m3": (c_int, [_P, _I, _L, _P, _P, _P, _P]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 

@@ -23,6 +23,7 @@ from typing import Optional
 
 import torch
 
+from . import _native as N
 from .flash_attn_interface import _flash_attn_backward, _flash_attn_forward, attn_bwd_block
 from .merge import (MAX_MERGE_MANY, get_default_args, grad_accumulate, merge_into, merge_many, pack_block,
                     update_out_and_lse)
@@ -269,12 +270,21 @@ def zigzag_causal_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=True
 
 
 def quantize_e4m3(x: torch.Tensor):
-    """Per-tensor e4m3 quantisation: scale s = amax / 448 (fp32), x_q = round-to-nearest-even(x / s)."""
-    amax = x.abs().amax().to(torch.float32) if x.numel() else torch.zeros((), dtype=torch.float32, device=x.device)
-    # amax / 448 in fp64, rounded once to fp32: the same bits on the host and on the device
-    scale = torch.where(amax > 0, (amax.double() / 448.0).float(), torch.ones_like(amax))
-    xq = (x.to(torch.float32) / scale).clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
-    return xq, scale
+    """Per-tensor e4m3 quantisation through mhip_quantize_e4m3: scale s = amax / 448 (fp32; 1 for an all-zero
+    tensor), x_q = round-to-nearest-even(clamp(x / s, -448, 448)) as ``torch.float8_e4m3fn``.  Returns
+    ``(x_q, s)`` with ``s`` a 0-dim fp32 tensor on the device (the block kernel's descale).  fp32 or bf16
+    input on the GPU."""
+    N.require_cuda(x)
+    if x.dtype not in (torch.float32, torch.bfloat16):
+        raise RuntimeError("quantize_e4m3 takes float32 or bfloat16")
+    xc = x.contiguous()
+    xq = torch.empty(xc.shape, dtype=torch.float8_e4m3fn, device=x.device)
+    ws = torch.empty(2, dtype=torch.float32, device=x.device)          # [scale, scratch for the maximum]
+    with torch.cuda.device(x.device):
+        code = N.lib().mhip_quantize_e4m3(N.ptr(xc), N.MHIP_F32 if x.dtype == torch.float32 else N.MHIP_BF16,
+                                          xc.numel(), N.ptr(xq), ws.data_ptr(), ws.data_ptr() + 4, N.stream_of(xc))
+    N.check(code, "mhip_quantize_e4m3")
+    return xq, ws[0]
 
 
 def fp8_pack_split_kv(q, kv, o, lse, softmax_scale, q_descale, k_descale, v_descale, dropout_p=0,
