@@ -168,6 +168,14 @@ int mhip_pack_reduce(const float* lhs, const void* block_out, const float* block
                      float* dst, int B, int Sq, int Hq, int D, void* stream);
 
 /*
+ * Epilogue of the packed form.  Replaces `o[...] = buf[..., :-1].to(q.dtype)` and
+ * `lse[...] = buf[..., -1].transpose(1, 2)` (the stores after the managed reduction,
+ * utils/flash_attn_dsl.py:406-407): buf fp32 (B,Sq,Hq,D+1) contiguous, out bf16 (B,Sq,Hq,D)
+ * contiguous and 16-byte aligned, lse fp32 (B,Hq,Sq) contiguous.  D a multiple of 8 that divides 2048.
+ */
+int mhip_unpack(const float* buf, void* out, float* lse, int B, int Sq, int Hq, int D, void* stream);
+
+/*
  * Gradient accumulation `torch.add(buf, block.to(float32))` (utils/attn_bwd_dsl.py:117-129):
  * dst = (acc ? acc : 0) + float(block), n elements, block in bf16; dst may alias acc.
  */

@@ -12,7 +12,7 @@ from .flash_attn_interface import (_flash_attn_backward, _flash_attn_forward, at
                                    attn_fwd_block)
 from .graph import GraphedStep
 from .merge import (LocalGroup, _update_out_and_lse, add_collective, flash_reduce, get_default_args,
-                    grad_accumulate, merge_into, merge_many, pack_block, update_out_and_lse,
+                    grad_accumulate, merge_into, merge_many, pack_block, unpack_into, update_out_and_lse,
                     update_out_and_lse_collective)
 from .ring import (flash_attn_backward, flash_attn_expose_reduce, flash_attn_expose_reduce_q_ring,
                    flash_attn_pack_kv,

@@ -33,6 +33,7 @@ _SIGNATURES = {
     "mhip_flash_reduce": (c_int, [_P] * 3 + [_L, _I, _P]),
     "mhip_tree_merge": (c_int, [_P] * 3 + [_L, _I, _I, _P]),
     "mhip_pack_reduce": (c_int, [_P] * 4 + [_I] * 4 + [_P]),
+    "mhip_unpack": (c_int, [_P] * 3 + [_I] * 4 + [_P]),
     "mhip_grad_accumulate": (c_int, [_P] * 3 + [_L, _P]),
     "mhip_quantize_e4m3": (c_int, [_P, _I, _L, _P, _P, _P, _P]),
 }

@@ -411,6 +411,27 @@ __global__ __launch_bounds__(256) void pack_reduce_kernel(const float* __restric
   store4<IT>(dst, g, total, r);
 }
 
+// Epilogue of the packed form (utils/flash_attn_dsl.py:406-407 after the managed reduction: the output is
+// buf[..., :-1] cast to the query's type, the LSE buf[..., -1] transposed to (B,H,S)): one row per D/8 lanes,
+// eight 4-byte loads (a packed row starts on a 4-byte boundary only) and one 16-byte store per lane.
+__global__ __launch_bounds__(256) void unpack_kernel(const float* __restrict__ buf, uint16_t* __restrict__ out,
+                                                     float* __restrict__ lse, uint32_t rows, uint32_t D,
+                                                     uint32_t Sq, uint32_t Hq) {
+  const uint32_t lpr = D / 8;
+  const uint32_t row = (blockIdx.x * 256u + threadIdx.x) / lpr;
+  if (row >= rows) return;
+  const uint32_t col = ((blockIdx.x * 256u + threadIdx.x) % lpr) * 8;
+  const float* src = buf + (uint64_t)row * (D + 1) + col;
+  u32x4 w;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) w[j] = pack_bf16(src[2 * j], src[2 * j + 1]);
+  *reinterpret_cast<u32x4*>(out + (uint64_t)row * D + col) = w;
+  if (col == 0) {
+    const uint32_t h = row % Hq, bs = row / Hq, s = bs % Sq, b = bs / Sq;
+    lse[((uint64_t)b * Hq + h) * Sq + s] = buf[(uint64_t)row * (D + 1) + D];
+  }
+}
+
 // ---- all blocks of a step at once --------------------------------------------------------------------
 // The chunk loop of a ring step folds N block results into the accumulators one after the other
 // (utils/flash_attn_dsl.py:51-71 called once per chunk, then the stores of :178-179), which moves the fp32
@@ -692,6 +713,21 @@ extern "C" int mhip_pack_reduce(const float* lhs, const void* block_out, const f
   } else {
     hipLaunchKernelGGL((pack_reduce_kernel<false, 0, uint64_t>), grid, block, 0, st, lhs, bo, block_lse, dst, (uint64_t)total, w, sq, hq);
   }
+  return launch_status();
+}
+
+extern "C" int mhip_unpack(const float* buf, void* out, float* lse, int B, int Sq, int Hq, int D, void* stream) {
+  if (B < 0 || Sq < 0 || Hq < 0 || D <= 0) return MHIP_EINVAL;
+  if (D % 8 != 0 || 256 % (D / 8) != 0) return MHIP_EUNSUPPORTED;
+  const int64_t rows = (int64_t)B * Sq * Hq;
+  if (rows == 0) return MHIP_OK;
+  if (rows >= (int64_t(1) << 31) / (D / 8)) return MHIP_EUNSUPPORTED;
+  if (!buf || !out || !lse) return MHIP_EINVAL;
+  if (!aligned16(out) || (reinterpret_cast<uintptr_t>(buf) & 3u)) return MHIP_EALIGN;
+  const int64_t threads = rows * (D / 8);
+  hipLaunchKernelGGL(unpack_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), buf, static_cast<uint16_t*>(out), lse, (uint32_t)rows,
+                     (uint32_t)D, (uint32_t)Sq, (uint32_t)Hq);
   return launch_status();
 }
 

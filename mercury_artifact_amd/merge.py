@@ -15,7 +15,7 @@ import torch
 from . import _native as N
 
 __all__ = ["get_default_args", "update_out_and_lse", "_update_out_and_lse", "flash_reduce",
-           "pack_block", "merge_into", "merge_many", "grad_accumulate", "update_out_and_lse_collective", "add_collective",
+           "pack_block", "unpack_into", "merge_into", "merge_many", "grad_accumulate", "update_out_and_lse_collective", "add_collective",
            "LocalGroup"]
 
 
@@ -270,6 +270,23 @@ def pack_block(block_out: torch.Tensor, block_lse: torch.Tensor,
                                         B, Sq, Hq, D, N.stream_of(block_out))
     N.check(code, "mhip_pack_reduce")
     return dst
+
+
+def unpack_into(buf: torch.Tensor, out: torch.Tensor, lse: torch.Tensor) -> None:
+    """``out[...] = buf[..., :-1].to(out.dtype)``, ``lse[...] = buf[..., -1].transpose(1, 2)`` (the stores after
+    the managed reduction, utils/flash_attn_dsl.py:406-407) in one pass: buf (B,Sq,Hq,D+1) fp32, out
+    (B,Sq,Hq,D) bf16 contiguous, lse (B,Hq,Sq) fp32 contiguous."""
+    N.require_cuda(buf, out, lse)
+    B, Sq, Hq, W = buf.shape
+    D = W - 1
+    if buf.dtype != torch.float32 or out.shape != (B, Sq, Hq, D) or lse.shape != (B, Hq, Sq):
+        raise RuntimeError("unpack_into takes a float32 (B,Sq,Hq,D+1) buffer, out (B,Sq,Hq,D) and lse (B,Hq,Sq)")
+    if out.dtype != torch.bfloat16 or lse.dtype != torch.float32 or not (out.is_contiguous() and lse.is_contiguous()):
+        raise RuntimeError("out must be contiguous bfloat16 and lse contiguous float32")
+    buf = buf.contiguous()
+    with torch.cuda.device(buf.device):
+        code = N.lib().mhip_unpack(N.ptr(buf), N.ptr(out), N.ptr(lse), B, Sq, Hq, D, N.stream_of(buf))
+    N.check(code, "mhip_unpack")
 
 
 def grad_accumulate(acc: Optional[torch.Tensor], block: torch.Tensor) -> torch.Tensor:

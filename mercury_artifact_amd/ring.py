@@ -26,7 +26,7 @@ import torch
 from . import _native as N
 from .flash_attn_interface import _flash_attn_backward, _flash_attn_forward, attn_bwd_block
 from .merge import (MAX_MERGE_MANY, get_default_args, grad_accumulate, merge_into, merge_many, pack_block,
-                    update_out_and_lse)
+                    unpack_into, update_out_and_lse)
 from .schedule import (LocalRing, n_dim_to_one_dim, one_dim_to_n_dim, reduce_buffer_route, shift_tuple_element,
                        zigzag_step)
 
@@ -150,9 +150,20 @@ def flash_attn_pack_split_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=F
                   fused_epilogue, deferred_merge)
 
 
+def _store_packed(buf, o, lse, fused: bool):
+    """The stores after the managed reduction (utils/flash_attn_dsl.py:406-407): one kernel, or the literal
+    torch expressions."""
+    if fused and o.dtype == torch.bfloat16 and o.is_contiguous() and lse.is_contiguous() and o.shape[-1] % 8 == 0 \
+            and 256 % (o.shape[-1] // 8) == 0:
+        unpack_into(buf, o, lse)
+        return
+    o[:, :, :, :] = buf[..., :-1].to(o.dtype)
+    lse[:, :, :] = buf[..., -1].transpose(1, 2)
+
+
 def flash_attn_expose_reduce(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False,
                              window_size=(-1, -1), alibi_slopes=None, deterministic=False, *,
-                             ring: LocalRing):
+                             ring: LocalRing, fused_epilogue: bool = True):
     """Managed-reduction form (template utils/flash_attn_dsl.py:345-408) with the KV ring: block
     results are packed ``(out | lse)`` and folded by ``flash_reduce``; pack and reduce run as one
     kernel."""
@@ -174,13 +185,12 @@ def flash_attn_expose_reduce(q, kv, o, lse, softmax_scale, dropout_p=0, causal=F
         assert len(outputs) == 4
         block_out, block_lse, _, _ = outputs
         buf = pack_block(block_out, block_lse, reduce_into=buf)
-    o[:, :, :, :] = buf[..., :-1].to(o.dtype)
-    lse[:, :, :] = buf[..., -1].transpose(1, 2)
+    _store_packed(buf, o, lse, fused_epilogue)
 
 
 def flash_attn_expose_reduce_q_ring(qs, kvs, os_, lses, softmax_scale, dropout_p=0, causal=False,
                                     window_size=(-1, -1), alibi_slopes=None, deterministic=False, *,
-                                    mesh_shape=None):
+                                    mesh_shape=None, fused_epilogue: bool = True):
     """The managed-reduction template (utils/flash_attn_dsl.py:345-408) scheduled as a ring over the
     *reduce buffer*: every rank keeps its KV shard, Q and the packed partial result ``(out | lse)``
     travel (codegen.py:116-190).  A rank's step is: block forward of the Q that just arrived against
@@ -217,8 +227,7 @@ def flash_attn_expose_reduce_q_ring(qs, kvs, os_, lses, softmax_scale, dropout_p
             for r in range(world):
                 home[home_of[r]] = buf[r]
     for r in range(world):
-        os_[r][:, :, :, :] = home[r][..., :-1].to(os_[r].dtype)
-        lses[r][:, :, :] = home[r][..., -1].transpose(1, 2)
+        _store_packed(home[r], os_[r], lses[r], fused_epilogue)
 
 
 def zigzag_causal_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=True, window_size=(-1, -1),

@@ -97,6 +97,10 @@ def test_elementwise_rejects(lib):
     assert lib.mhip_grad_accumulate(None, P, None, 16, None) == EINVAL
     assert lib.mhip_grad_accumulate(None, P + 2, P, 16, None) == EALIGN
     assert lib.mhip_grad_accumulate(None, P, P, 0, None) == OK
+    assert lib.mhip_unpack(P, None, P, 1, 8, 2, 128, None) == EINVAL
+    assert lib.mhip_unpack(P, P + 8, P, 1, 8, 2, 128, None) == EALIGN
+    assert lib.mhip_unpack(P, P, P, 1, 8, 2, 100, None) == EUNSUPPORTED
+    assert lib.mhip_unpack(P, P, P, 0, 8, 2, 128, None) == OK
     assert lib.mhip_quantize_e4m3(P, 1, 64, P, P, P, None) == EDTYPE
     assert lib.mhip_quantize_e4m3(P, 2, -1, P, P, P, None) == EINVAL
     assert lib.mhip_quantize_e4m3(P, 2, 64, P, None, P, None) == EINVAL

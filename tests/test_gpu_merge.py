@@ -261,3 +261,20 @@ def test_merge_many_with_partial_row_ranges():
     assert torch.allclose(fl.cpu(), rl, atol=1e-5, rtol=1e-5)
     with pytest.raises(RuntimeError):
         M.merge_many([t.cuda() for t in outs], [t.cuda() for t in lses], fo, fl, row_begin=[0] * 6)
+
+
+@pytest.mark.parametrize("B,Sq,H,D", [(2, 37, 3, 128), (1, 5, 2, 64), (1, 300, 1, 256)])
+def test_unpack_matches_the_literal_epilogue(B, Sq, H, D):
+    """buf[..., :-1].to(bf16) and buf[..., -1].transpose(1, 2) in one kernel: bit-exact (a cast and a copy)."""
+    import mercury_artifact_amd as M
+
+    g = torch.Generator().manual_seed(B + Sq)
+    buf = torch.randn(B, Sq, H, D + 1, generator=g)
+    buf[0, 0, 0, -1] = -math.inf
+    o = torch.full((B, Sq, H, D), 3.0, dtype=torch.bfloat16, device="cuda")
+    lse = torch.full((B, H, Sq), 3.0, dtype=torch.float32, device="cuda")
+    M.unpack_into(buf.cuda(), o, lse)
+    assert torch.equal(o.cpu(), buf[..., :-1].bfloat16())
+    assert torch.equal(lse.cpu(), buf[..., -1].transpose(1, 2))
+    with pytest.raises(RuntimeError):
+        M.unpack_into(buf.cuda(), o.float(), lse)
