@@ -99,7 +99,8 @@ def test_double_ring(rank):
     _compare(o, lse, ro, rl)
 
 
-def test_packed_reduce_ring():
+@pytest.mark.parametrize("fused", [False, True])
+def test_packed_reduce_ring(fused):
     import mercury_artifact_amd as M
 
     B, S, H, D, W, rank = 2, 1024, 3, 128, 4, 1
@@ -109,7 +110,8 @@ def test_packed_reduce_ring():
     dev = [c.cuda() for c in kvs]
     o = torch.empty(B, S // W, H, D, dtype=torch.bfloat16, device="cuda")
     lse = torch.empty(B, H, S // W, dtype=torch.float32, device="cuda")
-    M.flash_attn_expose_reduce(qs[rank].cuda(), dev[rank], o, lse, scale, ring=M.LocalRing((W,), rank, dev))
+    M.flash_attn_expose_reduce(qs[rank].cuda(), dev[rank], o, lse, scale, ring=M.LocalRing((W,), rank, dev),
+                               fused_epilogue=fused)
     _compare(o, lse, ro, rl)
 
 
