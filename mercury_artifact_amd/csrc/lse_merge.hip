@@ -172,9 +172,10 @@ void launch_merge(const MergeParams& p, bool first, bool fin, hipStream_t st) {
 
 // The same merge with eight head-dim values per lane: one 16-byte load of the bf16 block row piece, two
 // 16-byte loads and stores of the fp32 accumulator.  Measured at 131072 rows x 128 against the kernel
-// above: 29.1 vs 30.5 us into a separate destination, 28.0 vs 29.2 us in place, 21.9 vs 29.8 us with the
-// fused bf16 epilogue; the first-call cast is faster with four values per lane (16.8 vs 21.1 us) and stays
-// there.  One row per thread is the fastest setting here.
+// above, launches back to back: 29.1 vs 30.5 us into a separate destination, 28.0 vs 29.2 us in place,
+// 21.9 vs 29.8 us with the fused bf16 epilogue, 21.1 vs 16.8 us for the first-call cast.  Inside a ring
+// step, where a merge follows a block forward and its operands were written just before, the plain merge
+// is faster with four values per lane (31.6 vs 33.4 us), so only the fused-epilogue merges run here.
 #ifndef MHIP_MERGE8_ROWS
 #define MHIP_MERGE8_ROWS 1
 #endif
@@ -584,7 +585,10 @@ extern "C" int mhip_lse_merge(const float* acc_out, const float* acc_lse,
   if (dst_out) vec = vec && mult4(do_sb) && mult4(do_ss) && mult4(do_sh) && aligned16(dst_out);
   if (fin) vec = vec && (reinterpret_cast<uintptr_t>(final_out) & 7u) == 0;
   auto mult8 = [](int64_t x) { return (x & 7) == 0; };
-  const bool vec8 = vec && !first && D == 128 && mult8(bo_sb) && mult8(bo_ss) && mult8(bo_sh) && aligned16(block_out) &&
+#ifndef MHIP_MERGE8
+#define MHIP_MERGE8 1      // 1: merges with the fused bf16 epilogue, 2: every merge but the first call, 0: none
+#endif
+  const bool vec8 = (MHIP_MERGE8 == 2 || (MHIP_MERGE8 == 1 && fin)) && vec && !first && D == 128 && mult8(bo_sb) && mult8(bo_ss) && mult8(bo_sh) && aligned16(block_out) &&
                     (!fin || aligned16(final_out));
   if (vec8) {
     launch_merge8<16>(p, first, fin, st);
