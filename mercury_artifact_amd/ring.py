@@ -81,73 +81,92 @@ def _fwd_params(q, k, v, softmax_scale, dropout_p, causal, window_size, alibi_sl
 
 
 def _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes,
-                  ring: LocalRing, fused_epilogue: bool, deferred_merge: bool, **extra):
+                  ring: LocalRing, fused_epilogue: bool, deferred_merge: bool, ring_divide: int = 1, **extra):
+    """The chunk loop of the forward templates.  ``ring_divide = k > 1`` is the schedule option of the same
+    name (mercury/backend/pytorch/codegen.py:299-306): an outer loop over k sub-chunks of the KV rows wraps
+    the ring loop, so the step makes k * W block calls on (Sq x Sc / k) blocks and every hop moves 1/k of a
+    chunk."""
     blocks = []
     _out = None
     _lse = None
     _kv = None
     _next_kv = None
     steps = list(_hops(ring))
-    defer = (deferred_merge and len(steps) <= MAX_MERGE_MANY and o.dtype == torch.bfloat16
+    ring_divide = int(ring_divide)
+    Sc = kv.shape[2]
+    if ring_divide < 1 or Sc % ring_divide:
+        raise ValueError("ring_divide must divide the chunk's rows")
+    if ring_divide > 1 and ring.chunks is None:
+        raise ValueError("ring_divide needs a LocalRing that holds the chunks")
+    sub = Sc // ring_divide
+    n_blocks = len(steps) * ring_divide
+    defer = (deferred_merge and n_blocks <= MAX_MERGE_MANY and o.dtype == torch.bfloat16
              and o.is_contiguous() and lse.is_contiguous())
-    for step, hop in enumerate(steps):
-        if step == 0:
-            _kv = kv.contiguous()
-        else:
-            ring.wait()
-            _kv = _next_kv
-        if hop is not None:
-            send_to, recv_from = _neighbours(ring, hop)
-            _next_kv = ring.send_recv(send_to, recv_from, _kv)
-            ring.commit()
-        _k = _kv[0]
-        _v = _kv[1]
-        outputs = _flash_attn_forward(**_fwd_params(q, _k, _v, softmax_scale, dropout_p, causal,
-                                                    window_size, alibi_slopes, **extra))
-        assert len(outputs) == 4
-        block_out, block_lse, _, _ = outputs
-        if defer:
-            blocks.append((block_out, block_lse))
-            if step + 1 == len(steps):
-                merge_many([b[0] for b in blocks], [b[1] for b in blocks], o, lse)
+    done = 0
+    for part in range(ring_divide):
+        rows = slice(part * sub, (part + 1) * sub)
+        part_ring = ring if ring_divide == 1 else \
+            LocalRing(ring.mesh_shape, ring.rank, [c[:, :, rows] for c in ring.chunks], copy=ring.copy)
+        for step, hop in enumerate(steps):
+            if step == 0:
+                _kv = kv[:, :, rows].contiguous()
+            else:
+                part_ring.wait()
+                _kv = _next_kv
+            if hop is not None:
+                send_to, recv_from = _neighbours(part_ring, hop)
+                _next_kv = part_ring.send_recv(send_to, recv_from, _kv)
+                part_ring.commit()
+            _k = _kv[0]
+            _v = _kv[1]
+            outputs = _flash_attn_forward(**_fwd_params(q, _k, _v, softmax_scale, dropout_p, causal,
+                                                        window_size, alibi_slopes, **extra))
+            assert len(outputs) == 4
+            block_out, block_lse, _, _ = outputs
+            done += 1
+            if defer:
+                blocks.append((block_out, block_lse))
+                if done == n_blocks:
+                    merge_many([b[0] for b in blocks], [b[1] for b in blocks], o, lse)
+                    return
+                continue
+            if fused_epilogue and done == n_blocks:
+                # last merge writes o / lse directly (same arithmetic, two passes fewer)
+                merge_into(_out, _lse, block_out, block_lse, None, None, o, lse)
                 return
-            continue
-        if fused_epilogue and step + 1 == len(steps):
-            # last merge writes o / lse directly (same arithmetic, two passes fewer)
-            merge_into(_out, _lse, block_out, block_lse, None, None, o, lse)
-            return
-        _out, _lse = update_out_and_lse(_out, _lse, block_out, block_lse)
+            _out, _lse = update_out_and_lse(_out, _lse, block_out, block_lse)
     o[:, :, :, :] = _out.to(o.dtype)
     lse[:, :, :] = _lse.squeeze(dim=-1).transpose(1, 2)
 
 
 def flash_attn_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False, window_size=(-1, -1),
                        alibi_slopes=None, deterministic=False, *, ring: LocalRing,
-                       fused_epilogue: bool = True, deferred_merge: bool = True):
+                       fused_epilogue: bool = True, deferred_merge: bool = True, ring_divide: int = 1):
     """Single-ring forward step (template utils/flash_attn_dsl.py:127-180).  q (B,Sq,H,D), kv the
     rank's own (2,B,Sc,H,D), o (B,Sq,H,D) and lse (B,H,Sq) are written."""
     _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes, ring,
-                  fused_epilogue, deferred_merge)
+                  fused_epilogue, deferred_merge, ring_divide)
 
 
 def gqa_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False, window_size=(-1, -1),
                 alibi_slopes=None, deterministic=False, *, ring: LocalRing, fused_epilogue: bool = True,
-                deferred_merge: bool = True):
+                deferred_merge: bool = True, ring_divide: int = 1):
     """GQA forward step (template utils/flash_attn_dsl.py:182-235): kv has Hkv heads, q has
     Hkv * HEADS_PER_GROUP; the block kernel maps q head h to kv head h // HEADS_PER_GROUP."""
     _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes, ring,
-                  fused_epilogue, deferred_merge)
+                  fused_epilogue, deferred_merge, ring_divide)
 
 
 def flash_attn_pack_split_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False,
                              window_size=(-1, -1), alibi_slopes=None, deterministic=False, *,
-                             ring: LocalRing, fused_epilogue: bool = True, deferred_merge: bool = True):
+                             ring: LocalRing, fused_epilogue: bool = True, deferred_merge: bool = True,
+                             ring_divide: int = 1):
     """Double-ring forward step (template utils/flash_attn_dsl.py:237-291): ``ring`` is built on the
     2-D mesh ``(inner, outer)``; the loop order and hops follow from the mesh shape."""
     if len(ring.mesh_shape) != 2:
         raise ValueError("the double ring needs a 2-D mesh (inner, outer)")
     _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes, ring,
-                  fused_epilogue, deferred_merge)
+                  fused_epilogue, deferred_merge, ring_divide)
 
 
 def _store_packed(buf, o, lse, fused: bool):
@@ -298,10 +317,12 @@ def quantize_e4m3(x: torch.Tensor):
 
 def fp8_pack_split_kv(q, kv, o, lse, softmax_scale, q_descale, k_descale, v_descale, dropout_p=0,
                       causal=False, window_size=(-1, -1), alibi_slopes=None, deterministic=False, *,
-                      ring: LocalRing, fused_epilogue: bool = True, deferred_merge: bool = True):
+                      ring: LocalRing, fused_epilogue: bool = True, deferred_merge: bool = True,
+                      ring_divide: int = 1):
     """Forward step on e4m3 Q/K/V with per-tensor descales (not in the reference); any mesh."""
     _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes, ring,
-                  fused_epilogue, deferred_merge, q_descale=q_descale, k_descale=k_descale, v_descale=v_descale)
+                  fused_epilogue, deferred_merge, ring_divide, q_descale=q_descale, k_descale=k_descale,
+                  v_descale=v_descale)
 
 
 def flash_attn_backward(q, kv, o, lse, dout, dq, dkv, softmax_scale, dropout_p=0, causal=False,

@@ -57,6 +57,47 @@ def test_single_ring_reference_test_shape(rank, fused, deferred):
     assert torch.equal(qd, q_before) and torch.equal(dev_kvs[rank], kv_before)   # inputs untouched
 
 
+@pytest.mark.parametrize("divide,deferred", [(2, True), (4, True), (4, False)])
+def test_single_ring_with_ring_divide(divide, deferred):
+    """ring_divide = k (tests/test_ring_attn_codegen.py:102, benchmark/bench_attn.py:178): k * W block calls on
+    sub-chunks in the order of the generated loops; the result is attention over all keys."""
+    import mercury_artifact_amd as M
+
+    B, S, H, D, W, rank = 2, 2048, 3, 128, 4, 3
+    q, k, v, qs, kvs = _inputs(B, S, H, H, D, W, seed=5)
+    scale = D ** -0.5
+    sub = S // W // divide
+    subchunks = {(c, s): kvs[c][:, :, s * sub:(s + 1) * sub].float() for c in range(W) for s in range(divide)}
+    order = O.ring_divide_order(rank, W, divide)
+    keys = list(subchunks)
+    ro, rl = O.ring_forward(qs[rank].float(), [subchunks[key] for key in keys], [keys.index(x) for x in order], scale)
+    so, sl = O.single_pass_attention(qs[rank].float(), k.float(), v.float(), scale)
+    assert torch.allclose(ro, so, atol=1e-5)
+    dev = [c.cuda() for c in kvs]
+    o = torch.empty(B, S // W, H, D, dtype=torch.bfloat16, device="cuda")
+    lse = torch.empty(B, H, S // W, dtype=torch.float32, device="cuda")
+    from mercury_artifact_amd import flash_attn_interface as FI
+
+    calls = []
+    real = FI.attn_fwd_block
+
+    def counted(q_, k_, *a, **kw):
+        calls.append(tuple(k_.shape))
+        return real(q_, k_, *a, **kw)
+
+    FI.attn_fwd_block = counted
+    try:
+        M.flash_attn_pack_kv(qs[rank].cuda(), dev[rank], o, lse, scale, ring=M.LocalRing((W,), rank, dev),
+                             ring_divide=divide, deferred_merge=deferred)
+    finally:
+        FI.attn_fwd_block = real
+    assert calls == [(B, sub, H, D)] * (W * divide)
+    _compare(o, lse, ro, rl)
+    with pytest.raises(ValueError):
+        M.flash_attn_pack_kv(qs[rank].cuda(), dev[rank], o, lse, scale, ring=M.LocalRing((W,), rank, dev),
+                             ring_divide=7)
+
+
 def test_gqa_ring():
     """Hq 32 / Hkv 8 (tests/test_gqa.py:25), shortened sequence."""
     import mercury_artifact_amd as M
