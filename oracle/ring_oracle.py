@@ -35,7 +35,7 @@ __all__ = [
     "update_out_and_lse", "merge_chain", "pack_block", "flash_reduce", "tree_merge", "block_backward",
     "single_ring_order", "double_ring_order", "ring_divide_order",
     "zigzag_blocks", "zigzag_step", "zigzag_local_positions",
-    "quantize_e4m3", "dequantize",
+    "quantize_e4m3", "dequantize", "e4m3_p_rounding_bound",
     "ring_forward", "ring_forward_packed", "ring_backward", "zigzag_ring_forward",
 ]
 
@@ -291,6 +291,16 @@ def dequantize(xq: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
 # --------------------------------------------------------------------------------------
 # ring-step drivers: the loop the code generator emits (mercury/backend/pytorch/codegen.py:264-355,
 # 443-523) with the send/recv replaced by indexing a list of chunks
+def e4m3_p_rounding_bound(q, k, v, softmax_scale, causal=False):
+    """Per-element bound on what rounding the softmax numerators P to e4m3 (three mantissa bits: relative
+    error at most 2^-4 per value) can do to ``out = sum_i P_i v_i / sum_i P_i`` when the denominator keeps
+    the unrounded values: ``|error| <= 2^-4 * sum_i w_i |v_i|`` with ``w`` the softmax weights, i.e. 2^-4
+    times attention over ``|v|``.  Used by the tests as the tolerance of the fp8 kernel against attention on
+    the de-quantised operands (few visible keys and large |v| make it larger than any fixed number)."""
+    amp, _ = block_attention(q, k, v.abs(), softmax_scale, causal=causal)
+    return amp * 2.0 ** -4
+
+
 # --------------------------------------------------------------------------------------
 def ring_forward(q, kv_chunks: Sequence[torch.Tensor], order: Iterable[int], softmax_scale,
                  causal=False, dtype=torch.float32, block_out_dtype: Optional[torch.dtype] = None,

@@ -25,12 +25,16 @@ def _quantised(B, Sq, Sc, Hq, Hkv, seed, D=128):
     return (q, k, v), (qq, kq, vq), (sq, sk, sv)
 
 
-def _check(out, lse, ref_a, ref_b, tag, check_b=True):
+def _check(out, lse, ref_a, ref_b, tag, p_bound, check_b=True):
+    """Against attention on the de-quantised operands (ref_a): per element within what rounding P to e4m3 can
+    do (p_bound = O.e4m3_p_rounding_bound) plus one bf16 rounding of the result and 2e-3; rel-L2 <= 6e-2;
+    LSE rel <= 1e-3.  Against attention on the un-quantised operands (ref_b): the stated max-abs 6e-2, at
+    key counts where averaging makes it meaningful."""
     out, lse = out.float().cpu(), lse.cpu()
     (oa, la), (ob, _) = ref_a, ref_b
     assert not torch.isnan(out).any(), tag
     assert torch.equal(torch.isinf(lse), torch.isinf(la)), tag
-    excess = ((out - oa).abs() - (3e-2 + 2 ** -4 * oa.abs())).max().item()
+    excess = ((out - oa).abs() - (p_bound + 2 ** -8 * oa.abs() + 2e-3)).max().item()
     assert excess <= 0, (tag, excess)
     if oa.norm().item() > 0:
         assert (out - oa).norm().item() / oa.norm().item() <= 6e-2, (tag, (out - oa).norm().item() / oa.norm().item())
@@ -62,7 +66,8 @@ def test_fp8_block_matches_oracle(B, Sq, Sc, Hq, Hkv, causal):
         q_descale=sq.cuda(), k_descale=sk.cuda(), v_descale=sv.cuda())
     torch.cuda.synchronize()
     assert out.dtype == torch.bfloat16 and lse.dtype == torch.float32
-    _check(out, lse, ref_a, ref_b, "fp8 block", check_b=Sc >= 1000)
+    p_bound = O.e4m3_p_rounding_bound(O.dequantize(qq, sq), O.dequantize(kq, sk), O.dequantize(vq, sv), scale, causal=causal)
+    _check(out, lse, ref_a, ref_b, "fp8 block", p_bound, check_b=Sc >= 1000)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -128,4 +133,5 @@ def test_fp8_double_ring(rank):
     M.fp8_pack_split_kv(qq[:, qs].cuda(), dev[rank], o, lse, scale, sq.cuda(), sk.cuda(), sv.cuda(),
                         ring=M.LocalRing((4, 2), rank, dev))
     torch.cuda.synchronize()
-    _check(o, lse, ref_a, ref_b, "fp8 double ring")
+    p_bound = O.e4m3_p_rounding_bound(O.dequantize(qq[:, qs], sq), O.dequantize(kq, sk), O.dequantize(vq, sv), scale)
+    _check(o, lse, ref_a, ref_b, "fp8 double ring", p_bound)

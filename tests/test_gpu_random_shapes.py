@@ -85,10 +85,11 @@ def test_random_fp8_forward(B, Sq, Sc, Hq, Hkv, causal):
                                 q_descale=sq.cuda(), k_descale=sk.cuda(), v_descale=sv.cuda())
     out, lse = out.float().cpu(), lse.cpu()
     assert torch.equal(torch.isinf(lse), torch.isinf(la))
-    # own per-element bound against attention on the de-quantised inputs: 4e-2 + 2^-4 |ref| (rows that see two or
-    # three keys of opposite sign can cancel in |ref| but not in the rounding error of P), inside the stated
-    # fp8 bar of 6e-2
-    assert ((out - oa).abs() - (4e-2 + 2 ** -4 * oa.abs())).max().item() <= 0
+    # per element within what rounding P to e4m3 can do (2^-4 times attention over |v|: few visible keys and
+    # large |v| make that larger than any fixed number) plus one bf16 rounding of the result and 2e-3
+    p_bound = O.e4m3_p_rounding_bound(O.dequantize(qq, sq), O.dequantize(kq, sk), O.dequantize(vq, sv), scale,
+                                      causal=causal)
+    assert ((out - oa).abs() - (p_bound + 2 ** -8 * oa.abs() + 2e-3)).max().item() <= 0
     if oa.norm().item() > 0:
         assert (out - oa).norm().item() / oa.norm().item() <= 6e-2
     fin = ~torch.isinf(la)
