@@ -132,7 +132,7 @@ int mhip_lse_merge_many(const void* const* block_outs, const float* const* block
 /*
  * Packed merge.  Replaces TorchScript `flash_reduce` (utils/flash_attn_dsl.py:293-305):
  * lhs, rhs, dst are contiguous fp32 (rows, D+1), 16-byte aligned; dst must not overlap lhs
- * or rhs (the reference's flash_reduce returns a new tensor as well).
+ * or rhs (MHIP_EINVAL; the reference's flash_reduce returns a new tensor as well).
  */
 int mhip_flash_reduce(const float* lhs, const float* rhs, float* dst,
                       int64_t rows, int D, void* stream);
@@ -142,7 +142,8 @@ int mhip_flash_reduce(const float* lhs, const float* rhs, float* dst,
  * the caller).  With row_max[r] = max over ranks of the lse column (one MAX all-reduce of `rows` floats):
  *   finish == 0:  dst = (out * d | d), d = exp(lse - row_max)   -- this rank's term of ONE SUM all-reduce
  *   finish != 0:  src is the summed terms; dst = (sum_out / sum_d | row_max + log(sum_d))
- * dst may alias src.  Rows with row_max = -inf come out as (0 | -inf). */
+ * dst may be src itself (in place; any other overlap of the two is rejected with MHIP_EINVAL).  Rows with
+ * row_max = -inf come out as (0 | -inf). */
 int mhip_tree_merge(const float* src, const float* row_max, float* dst, int64_t rows, int D, int finish,
                     void* stream);
 
@@ -161,7 +162,7 @@ int mhip_quantize_e4m3(const void* x, int dtype, int64_t n, void* xq, float* sca
  * Pack a block result: dst (B,Sq,Hq,D+1) fp32 contiguous =
  * cat([float(block_out), block_lse^T], -1)   (utils/flash_attn_dsl.py:396).
  * If lhs is not NULL the pack is fused with the reduce: dst = flash_reduce(lhs, pack(block));
- * dst must not overlap lhs; dst and lhs 16-byte aligned.  block_out (B,Sq,Hq,D) bf16 and block_lse
+ * dst must not overlap lhs (MHIP_EINVAL); dst and lhs 16-byte aligned.  block_out (B,Sq,Hq,D) bf16 and block_lse
  * (B,Hq,Sq) contiguous.
  */
 int mhip_pack_reduce(const float* lhs, const void* block_out, const float* block_lse,

@@ -11,8 +11,7 @@
 //                a row XOR-swizzled, four stages each; every wavefront copies 8 rows of each tile
 //   S^T = K Q^T  : v_mfma_f32_32x32x16_bf16 with A = K rows (LDS), B = Q (registers, loaded once).
 //                  The accumulator layout puts one Q row in each lane (lane % 32) and 32 of the
-//                  64 keys of the tile in that lane's registers, so the online softmax needs one
-//                  exchange with lane ^ 32 per tile and no other cross-lane traffic.
+//                  64 keys of the tile in that lane's registers, so the softmax is lane-local.
 //   O^T = V^T P^T: the same lane that produced P^T[key][q] feeds it back as the B operand; the
 //                  key order inside one MFMA k-step is whatever the accumulator registers hold, and
 //                  the V^T operand is gathered in exactly that order from the row-major V tile by
@@ -21,6 +20,10 @@
 //                  32 MFMAs) and a vector phase (softmax of the next tile, tile copies).  Wavefronts
 //                  0-3 and 4-7 run half a tile apart, separated by workgroup barriers, so on every
 //                  SIMD one wavefront feeds the matrix pipe while the other does exponentials.
+//   softmax      : the reference score of a row is fixed by the first tile's row maximum and moves only
+//                  when a later tile would overflow: the row SUMS are watched (one compare per tile),
+//                  not the maxima, so the common path has no maximum, no cross-lane exchange and no
+//                  rescale of O; the matrix phase carries no vector work of its own.
 #include "mhip_common.hpp"
 
 namespace mhip {
@@ -171,28 +174,26 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 16; ++j) o_acc[i][j] = 0.f;
-  // m_ref: the score (raw, unscaled) the exponentials of this lane's Q row are taken relative to.  It
-  // follows the running maximum lazily: it only moves when the maximum has grown by more than
-  // kRescaleSlack (in log2 units of the scaled score), so exp2 arguments stay below that slack and the
-  // O accumulator is rescaled on few tiles.  The LSE does not depend on the choice of reference.
-  float m_ref = -INFINITY;
+  // m_ref: the raw (unscaled) score the exponentials of this lane's Q row are taken relative to.  It is
+  // fixed by the first tile's row maximum and moves only when a later tile would overflow: the row sums are
+  // watched, not the maxima, so the common path has no maximum, no cross-lane exchange and no rescale of O.
+  float m_ref = 0.f;
+  float nmsc = 0.f;          // -m_ref * scale * log2(e)
   float l_run = 0.f;         // this lane's share of the running sum (the other 32 keys: lane ^ 32)
-  constexpr float kRescaleSlack = 8.f;
+  constexpr float kTrigger = 1048576.f;   // a lane's 32 exponentials of one tile sum to less than this, or
+  constexpr float kSlack = 14.f;          // rows whose maximum exceeds the reference by 2^kSlack move it
+  const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   f32x16 s[2];               // S^T tile: 64 keys x 32 q rows per wave
   bf16x8 pf[4];              // P^T of the current tile as bf16 B operands
 
   auto qk = [&](int stage) {
     const unsigned char* ks = smem + stage * kTileBytes;
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-      for (int j = 0; j < 16; ++j) s[mb][j] = 0.f;
-#pragma unroll
     for (int kk = 0; kk < 8; ++kk) {
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb) {
         const bf16x8 kf = read_k(ks, mb, kk);
-        s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], s[mb], 0, 0, 0);
+        s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], kk == 0 ? zero : s[mb], 0, 0, 0);
       }
     }
   };
@@ -209,10 +210,6 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     }
   };
 
-  // ---- online softmax of one S^T tile (per lane = per Q row) -> pf, cut into pieces ---------------------
-  // The first kEarly exponentials are computed inside the matrix phase, behind the O^T MFMAs; the rest,
-  // the packing to bf16 and the (rare) rescale of O in the vector phase.  State shared by the pieces:
-  float mx = -INFINITY, msc = 0.f, rs = 0.f, alpha = 1.f;
   // keys past the chunk end and the causal diagonal -> -inf
   auto sm_mask = [&](int t) {
     const int kv0 = t * kBN;
@@ -230,68 +227,55 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
         }
     }
   };
-  // running maximum over accumulator registers 8i .. 8i+7 (i = 0..3)
-  auto sm_max = [&](int i) {
-    const int mb = i >> 1, base = (i & 1) * 8;
-    if (i == 0) mx = s[0][0];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) mx = fmaxf(mx, s[mb][base + j]);
-  };
-  // Combine with the other 32 keys and move the reference when the maximum outgrew it by the slack
-  // (always on the first tile with a visible key: m_ref = -inf there).  The factor alpha that O and the
-  // running sum owe to the move is applied later, by sm_finish, once the MFMAs of the tile before have
-  // landed in O.
-  auto sm_reference = [&]() {
-    mx = pair_max(mx);
-    const bool grow = (mx - m_ref) * p.scale_log2 > kRescaleSlack;     // false for NaN (-inf - -inf)
-    const float m_new = grow ? mx : m_ref;
-    alpha = (grow && m_new != -INFINITY) ? fast_exp2((m_ref - m_new) * p.scale_log2) : 1.f;
-    m_ref = m_new;
-    msc = (m_ref == -INFINITY) ? 0.f : m_ref * p.scale_log2;
+  // exponentials of the tile, P^T as bf16 B operands (k-step (mb, j2) takes accumulator registers
+  // 8 j2 .. 8 j2 + 7) and this lane's sum of them; s stays intact
+  float rs = 0.f;
+  auto sm_exps = [&]() {
     rs = 0.f;
-  };
-  // exponentials of accumulator registers 2e, 2e+1 (e = 0..15, counted over both 32-key blocks)
-  auto sm_exp = [&](int e) {
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int j = 2 * e + u;
-      const float x = fast_exp2(__builtin_fmaf(s[j >> 4][j & 15], p.scale_log2, -msc));
-      s[j >> 4][j & 15] = x;
-      rs += x;
-    }
-  };
-  // rescale (only if some row of the wave moved its reference), running sum, P^T as bf16 B operands:
-  // k-step (mb, j2) takes accumulator registers 8 j2 .. 8 j2 + 7
-  auto sm_finish = [&]() {
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
-#pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) o_acc[db][j] *= alpha;
-    }
-    l_run = l_run * alpha + rs;
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
       for (int j2 = 0; j2 < 2; ++j2) {
         u32x4 w;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) w[e] = pack_bf16(s[mb][8 * j2 + 2 * e], s[mb][8 * j2 + 2 * e + 1]);
+        for (int e = 0; e < 4; ++e) {
+          const float x0 = fast_exp2(__builtin_fmaf(s[mb][8 * j2 + 2 * e], p.scale_log2, nmsc));
+          const float x1 = fast_exp2(__builtin_fmaf(s[mb][8 * j2 + 2 * e + 1], p.scale_log2, nmsc));
+          w[e] = pack_bf16(x0, x1);
+          rs += x0 + x1;
+        }
         pf[mb * 2 + j2] = __builtin_bit_cast(bf16x8, w);
       }
   };
-#ifndef MHIP_FWD_EARLY
-#define MHIP_FWD_EARLY 10
-#endif
-  constexpr int kEarly = MHIP_FWD_EARLY;     // pairs of exponentials done in the matrix phase (slots 22..31)
-  auto softmax_all = [&](int t) {
-    sm_mask(t);
+  // Move the reference of the rows whose scores outgrew it (first tile: set it to the row maximum) and
+  // rescale O and the running sum accordingly.
+  auto sm_fix = [&](bool first) {
+    float mx = s[0][0];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) sm_max(i);
-    sm_reference();
+    for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) sm_exp(e);
-    sm_finish();
+      for (int j = 0; j < 16; ++j) mx = fmaxf(mx, s[mb][j]);
+    mx = pair_max(mx);
+    const float grown = (mx - m_ref) * p.scale_log2;               // NaN when mx = -inf on the first tile
+    const bool move = first ? (mx != -INFINITY) : (grown > kSlack);   // false for NaN
+    if (!first) {
+      const float alpha = move ? fast_exp2(-grown) : 1.f;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) o_acc[db][j] *= alpha;
+      l_run *= alpha;
+    }
+    m_ref = move ? mx : m_ref;
+    nmsc = -m_ref * p.scale_log2;
+  };
+  auto sm_tile = [&]() {
+    sm_exps();
+    if (__builtin_amdgcn_ballot_w64(!(rs < kTrigger)) != 0) {
+      sm_fix(false);
+      sm_exps();
+    }
+    l_run += rs;
   };
 
   // Matrix phase of tile t: S^T(t+1) from K stage `ks_stage` and O^T += V^T(t) P^T(t) from V stage
@@ -312,7 +296,6 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
   auto matrix_phase = [&](int t_next, int ks_stage, int vs_stage) {
     const unsigned char* ks = smem + ks_stage * kTileBytes;
     const unsigned char* vs = smem + kVBase + vs_stage * kTileBytes;
-    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
       if (i < 16) {
@@ -325,9 +308,6 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
       if (i + kFragDepth < 32) frag[i % kFragDepth] = read_frag(i + kFragDepth, ks, vs);
       // S^T(t_next) is complete after slot 15; its softmax starts here, in the shadow of the O^T MFMAs
       if (i == 16) sm_mask(t_next);
-      if (i >= 17 && i < 21) sm_max(i - 17);
-      if (i == 21) sm_reference();
-      if (i >= 22 && i - 22 < kEarly) sm_exp(i - 22);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -354,7 +334,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     qk(0);
-    softmax_all(0);
+    sm_mask(0);
+    sm_fix(true);
+    sm_exps();
+    l_run = rs;
     if (ntiles > 1) first_frags(1);
   }
   // Phase p of the main loop: group A (waves 0-3) runs the matrix phase of tile p/2 on even p and its
@@ -370,10 +353,9 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     matrix_phase(t + 1, (t + 1) & 3, t & 3);
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_s_barrier();
-    // ---- vector phase: rest of softmax(t+1), copies of the tiles ahead -------------------------------------
-#pragma unroll
-    for (int e = kEarly; e < 16; ++e) sm_exp(e);
-    sm_finish();
+    // ---- vector phase: softmax(t+1), copies of the tiles ahead ---------------------------------------------
+    asm volatile("" : "+v"(s[0]), "+v"(s[1]));      // keeps the exponentials behind the barrier
+    sm_tile();
     copy_k(t + 4, t & 3);
     copy_v(t + 3, (t + 3) & 3);
     if (t + 2 < ntiles) first_frags((t + 2) & 3);             // K(t+2), for the next matrix phase

@@ -125,34 +125,39 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const MergeParams p) {
   }
 }
 
-// Generic head dimension: one thread per (row, 4-element group) is replaced by one thread per
-// element; used only when D is not 32 / 64 / 128 / 256.
+// Generic head dimension or unaligned operands: one row per 32 lanes of one wavefront, the lanes stepping
+// through the columns.  dst may alias acc: an output element is read and written by the same lane only, and
+// the row's lse is loaded by all lanes of the row in one instruction before the one lane that owns it stores
+// the new value, which depends on that load (so the load has returned for the whole wavefront).
+constexpr int kGenericLanes = 32;
 template <bool FIRST, bool FINAL>
 __global__ __launch_bounds__(256) void lse_merge_generic(const MergeParams p, int D) {
-  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (e >= p.rows * D) return;
-  const int64_t row = e / D;
-  const int col = (int)(e % D);
+  const int64_t row = (int64_t)blockIdx.x * (256 / kGenericLanes) + threadIdx.x / kGenericLanes;
+  if (row >= p.rows) return;
+  const int lane = threadIdx.x % kGenericLanes;
   const int h = (int)(row % p.Hq);
   const int64_t bs = row / p.Hq;
   const int s = (int)(bs % p.Sq);
   const int b = (int)(bs / p.Sq);
-  const float bo = bf16_lo(p.block_out[b * p.bo_sb + s * p.bo_ss + h * p.bo_sh + col]);
   const float bl = p.block_lse[b * p.bl_sb + h * p.bl_sh + s];
-  float res = bo, new_lse = bl;
-  if (!FIRST) {
-    const float a = p.acc_out[b * p.ao_sb + s * p.ao_ss + h * p.ao_sh + col];
-    float w;
-    merge_weights(p.acc_lse[b * p.al_sb + s * p.al_ss + h * p.al_sh], bl, w, new_lse);
-    res = a - w * (a - bo);
+  float w = 1.f, new_lse = bl;
+  if (!FIRST) merge_weights(p.acc_lse[b * p.al_sb + s * p.al_ss + h * p.al_sh], bl, w, new_lse);
+  const uint16_t* bo_row = p.block_out + b * p.bo_sb + s * p.bo_ss + h * p.bo_sh;
+  const float* a_row = FIRST ? nullptr : p.acc_out + b * p.ao_sb + s * p.ao_ss + h * p.ao_sh;
+  float* d_row = p.dst_out ? p.dst_out + b * p.do_sb + s * p.do_ss + h * p.do_sh : nullptr;
+  for (int col = lane; col < D; col += kGenericLanes) {
+    const float bo = bf16_lo(bo_row[col]);
+    float res = bo;
+    if (!FIRST) {
+      const float a = a_row[col];
+      res = a - w * (a - bo);
+    }
+    if (d_row) d_row[col] = res;
+    if (FINAL) p.final_out[row * D + col] = (uint16_t)(pack_bf16(res, 0.f) & 0xffffu);
   }
-  if (p.dst_out != nullptr) {
-    p.dst_out[b * p.do_sb + s * p.do_ss + h * p.do_sh + col] = res;
-    if (col == 0) p.dst_lse[b * p.dl_sb + s * p.dl_ss + h * p.dl_sh] = new_lse;
-  }
-  if (FINAL) {
-    p.final_out[row * D + col] = (uint16_t)(pack_bf16(res, 0.f) & 0xffffu);
-    if (col == 0) p.final_lse[((int64_t)b * p.Hq + h) * p.Sq + s] = new_lse;
+  if (lane == 0) {
+    if (d_row) p.dst_lse[b * p.dl_sb + s * p.dl_ss + h * p.dl_sh] = new_lse;
+    if (FINAL) p.final_lse[((int64_t)b * p.Hq + h) * p.Sq + s] = new_lse;
   }
 }
 
@@ -365,6 +370,30 @@ __global__ __launch_bounds__(256) void tree_merge_kernel(const float* __restrict
     r[j] = cc == W - 1 ? last[k] : a[j] * f[k];
   }
   store4<IT>(dst, g, total, r);
+}
+
+// The same for dst == src (the natural use: all-reduce the packed buffer in place, finish in place).  The
+// flat walk above reads a row's last column from a thread that does not own it, so in place it would race
+// with the owner's store; here one row belongs to 32 lanes of one wavefront, which all load the last column
+// in one instruction before the lane that owns it stores the new value computed from that load.
+template <bool FINISH>
+__global__ __launch_bounds__(256) void tree_merge_rows_kernel(const float* src, const float* __restrict__ aux,
+                                                              float* dst, int64_t rows, uint32_t W) {
+  const int64_t row = (int64_t)blockIdx.x * (256 / kGenericLanes) + threadIdx.x / kGenericLanes;
+  if (row >= rows) return;
+  const uint32_t lane = threadIdx.x % kGenericLanes;
+  const float m = aux[row];
+  const float tail = src[row * W + W - 1];
+  float f, last;
+  if (!FINISH) {
+    f = (m == -INFINITY) ? 0.f : __expf(tail - m);
+    last = f;
+  } else {
+    f = tail > 0.f ? 1.f / tail : 0.f;
+    last = tail > 0.f ? m + __logf(tail) : -INFINITY;
+  }
+  for (uint32_t c = lane; c + 1 < W; c += kGenericLanes) dst[row * W + c] = src[row * W + c] * f;
+  if (lane == 0) dst[row * W + W - 1] = last;
 }
 
 template <bool REDUCE, int WCT, typename IT>
@@ -600,8 +629,9 @@ extern "C" int mhip_lse_merge(const float* acc_out, const float* acc_lse,
       default: launch_merge<64>(p, first, fin, st); break;
     }
   } else {
-    const int64_t n = p.rows * D;
-    const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    constexpr int kRowsPerBlock = 256 / kGenericLanes;
+    if (p.rows / kRowsPerBlock >= (int64_t(1) << 31)) return MHIP_EUNSUPPORTED;
+    const dim3 grid((unsigned)((p.rows + kRowsPerBlock - 1) / kRowsPerBlock)), block(256);
     if (first && fin) hipLaunchKernelGGL((lse_merge_generic<true, true>), grid, block, 0, st, p, D);
     else if (first) hipLaunchKernelGGL((lse_merge_generic<true, false>), grid, block, 0, st, p, D);
     else if (fin) hipLaunchKernelGGL((lse_merge_generic<false, true>), grid, block, 0, st, p, D);
@@ -654,6 +684,7 @@ extern "C" int mhip_flash_reduce(const float* lhs, const float* rhs, float* dst,
   if (!lhs || !rhs || !dst) return MHIP_EINVAL;
   if (!aligned16(lhs) || !aligned16(rhs) || !aligned16(dst)) return MHIP_EALIGN;
   const int64_t total = rows * (D + 1);
+  if ((dst < lhs + total && lhs < dst + total) || (dst < rhs + total && rhs < dst + total)) return MHIP_EINVAL;
   const int64_t groups = (total + 3) / 4;
   const dim3 grid((unsigned)((groups + 255) / 256)), block(256);
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -678,6 +709,15 @@ extern "C" int mhip_tree_merge(const float* src, const float* row_max, float* ds
   const dim3 grid((unsigned)((groups + 255) / 256)), block(256);
   hipStream_t st = static_cast<hipStream_t>(stream);
   const uint32_t w = (uint32_t)(D + 1);
+  if (dst == src) {
+    constexpr int kRowsPerBlock = 256 / kGenericLanes;
+    if (rows / kRowsPerBlock >= (int64_t(1) << 31)) return MHIP_EUNSUPPORTED;
+    const dim3 rgrid((unsigned)((rows + kRowsPerBlock - 1) / kRowsPerBlock));
+    if (finish) hipLaunchKernelGGL(tree_merge_rows_kernel<true>, rgrid, block, 0, st, src, row_max, dst, rows, w);
+    else hipLaunchKernelGGL(tree_merge_rows_kernel<false>, rgrid, block, 0, st, src, row_max, dst, rows, w);
+    return launch_status();
+  }
+  if (dst < src + total && src < dst + total) return MHIP_EINVAL;      // partial overlap
   if (total < (int64_t(1) << 31)) {
     const uint32_t t32 = (uint32_t)total;
     if (finish && D == 128) hipLaunchKernelGGL((tree_merge_kernel<true, 129, uint32_t>), grid, block, 0, st, src, row_max, dst, t32, w);
@@ -705,6 +745,7 @@ extern "C" int mhip_pack_reduce(const float* lhs, const void* block_out, const f
   hipStream_t st = static_cast<hipStream_t>(stream);
   const uint16_t* bo = static_cast<const uint16_t*>(block_out);
   if (lhs && !aligned16(lhs)) return MHIP_EALIGN;
+  if (lhs && dst < lhs + total && lhs < dst + total) return MHIP_EINVAL;
   const uint32_t w = (uint32_t)(D + 1), sq = (uint32_t)Sq, hq = (uint32_t)Hq;
   if (total < (int64_t(1) << 31)) {
     const uint32_t t32 = (uint32_t)total;

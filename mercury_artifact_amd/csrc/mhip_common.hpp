@@ -74,6 +74,10 @@ __device__ __forceinline__ u32x4 rsrc_words(const void* base, uint32_t bytes) {
 // offset is out of the descriptor's range write zeros.  Completion is counted by vmcnt.  Written as
 // inline assembly so that the compiler's own wait-count insertion does not see the copies: it would
 // otherwise wait for all of them before every transposing LDS read.  The kernels place the waits by hand.
+// M0 is written here and is not on the clobber list: the compiler treats it as a reserved register, warns
+// that a clobber of it "may not be preserved" and ignores it.  That is safe as long as nothing else in a
+// kernel that copies this way needs M0 (no register-indexed moves, no s_sendmsg, no GWS, no other LDS-direct
+// load): every copy sets M0 itself immediately before its load, so it never relies on an earlier value.
 __device__ __forceinline__ void copy16_to_lds(u32x4 rsrc, uint32_t lds_addr, int voffset, int soffset) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voffset), "s"(rsrc),

@@ -91,6 +91,13 @@ def test_elementwise_rejects(lib):
     assert lib.mhip_tree_merge(P, None, P, 8, 128, 0, None) == EINVAL
     assert lib.mhip_tree_merge(P + 8, P, P, 8, 128, 1, None) == EALIGN
     assert lib.mhip_tree_merge(P, P, P, 0, 128, 1, None) == OK
+    # overlapping operands: dst == src is the in-place form of the tree merge, any other overlap is refused;
+    # the flat packed kernels take no overlap at all
+    assert lib.mhip_tree_merge(P, P, P + 16, 8, 128, 1, None) == EINVAL
+    assert lib.mhip_tree_merge(P + 16, P, P, 8, 128, 0, None) == EINVAL
+    assert lib.mhip_flash_reduce(P, P + 0x100000, P, 8, 128, None) == EINVAL
+    assert lib.mhip_flash_reduce(P + 0x100000, P, P + 16, 8, 128, None) == EINVAL
+    assert lib.mhip_pack_reduce(P, P, P, P + 32, 1, 8, 2, 128, None) == EINVAL
     assert lib.mhip_pack_reduce(None, P, P, None, 1, 8, 2, 128, None) == EINVAL
     assert lib.mhip_pack_reduce(P + 4, P, P, P, 1, 8, 2, 128, None) == EALIGN
     assert lib.mhip_pack_reduce(None, P, P, P, 0, 8, 2, 128, None) == OK

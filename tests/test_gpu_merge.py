@@ -53,6 +53,45 @@ def test_update_out_and_lse_matches_reference_formula(B, Sq, H, D):
         M.update_out_and_lse(None, None, bod, bld, slice_=(slice(None), slice(0, 1)))
 
 
+@pytest.mark.parametrize("D", [40, 130])
+def test_merge_in_place_generic_head_dim_beyond_residency(D):
+    """dst == acc on the path taken for head dimensions other than 32/64/128/256 (one row per 32 lanes of one
+    wavefront: the row's lse is read by all its lanes before the one store), at a row count whose grid is far
+    larger than what is resident at once, so that rows merged late would see lse values stored early if any
+    thread read an lse it does not own."""
+    import mercury_artifact_amd as M
+
+    B, Sq, H = 2, 40000, 3
+    out, lse, bo, bl = _blocks(B, Sq, H, D, seed=3)
+    ro, rl = O.merge_reference(out, lse, bo, bl)
+    od, ld = out.cuda(), lse.cuda()
+    M.merge_into(od, ld, bo.cuda(), bl.cuda(), od, ld)                     # through mhip_lse_merge, dst = acc
+    torch.cuda.synchronize()
+    assert torch.allclose(od.cpu(), ro, **TOL) and torch.allclose(ld.cpu(), rl, **TOL)
+
+
+@pytest.mark.parametrize("D", [128, 24])
+def test_tree_merge_in_place(D):
+    """mhip_tree_merge with dst == src (both phases) equals the out-of-place result bit for bit."""
+    from mercury_artifact_amd import merge as MM
+
+    torch.manual_seed(11)
+    rows = 50001
+    src = torch.randn(rows, D + 1).cuda()
+    src[7, -1] = -math.inf
+    row_max = (src[:, -1] + torch.rand(rows).cuda()).contiguous()
+    row_max[7] = -math.inf
+    for finish in (False, True):
+        x = src.abs() if finish else src                                  # finish expects sum_d > 0 in the last column
+        sep = torch.empty_like(x)
+        MM._tree_merge(x, row_max, sep, finish)
+        inplace = x.clone()
+        MM._tree_merge(inplace, row_max, inplace, finish)
+        torch.cuda.synchronize()
+        assert torch.equal(sep.isnan(), inplace.isnan())
+        assert torch.equal(sep.nan_to_num(), inplace.nan_to_num())
+
+
 def test_merge_fused_final_epilogue():
     import mercury_artifact_amd as M
 
