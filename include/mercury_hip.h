@@ -3,8 +3,9 @@
  *
  * One shared library, libmercury_hip.so, plain pointers and sizes only.  Every pointer
  * is a DEVICE pointer unless stated otherwise; `stream` is a hipStream_t passed as
- * void* (NULL = the default stream).  All calls are asynchronous on `stream`, keep no
- * global mutable state and allocate nothing.  Return value: 0 on success, a negative
+ * void* (NULL = the default stream).  All calls are asynchronous on `stream`, allocate
+ * nothing and keep no global mutable state (mhip_attn_bwd_block_noalloc excepted: it owns
+ * a scratch array on every GPU).  Return value: 0 on success, a negative
  * MHIP_E* code otherwise (mhip_error_string() gives the text).  Nothing throws.
  *
  * Tensor layouts follow the call sites of the reference (paths relative to the
@@ -32,6 +33,8 @@ extern "C" {
 #define MHIP_EALIGN         -4   /* pointer or stride not 16-byte aligned              */
 #define MHIP_ELAUNCH        -5   /* hipLaunchKernel / hipGetLastError reported failure */
 #define MHIP_EUNSUPPORTED   -6   /* feature not implemented (dropout, alibi, window..) */
+#define MHIP_ETOOLARGE      -7   /* problem exceeds the built-in scratch of a *_noalloc entry point */
+#define MHIP_ERUNTIME       -8   /* a HIP runtime query (device, symbol address) failed */
 
 /* ---- element types -------------------------------------------------------------- */
 #define MHIP_BF16  0
@@ -82,6 +85,26 @@ int mhip_attn_bwd_block(const void* dout, const void* q, const void* k, const vo
                         int64_t dk_sb, int64_t dk_ss, int64_t dk_sh,  /* dk, dv          */
                         float softmax_scale, int mask, int deterministic,
                         void* workspace, void* stream);
+
+/*
+ * mhip_attn_bwd_block without the workspace argument.  No counterpart in the reference: it is for callers
+ * that cannot hand over (or allocate) scratch memory -- code under HIP graph capture, serving loops and
+ * harnesses that forbid hipMalloc.  delta and lse2 go to an array built into the library (a file-scope
+ * __device__ array of 8 MiB + 32 bytes, held by every GPU the library runs on until the process ends), so
+ * the block is limited to B * Hq * Sq <= 1048576 (MHIP_ETOOLARGE beyond).  The first call on a device asks
+ * the runtime for that device's address of the array (hipGetSymbolAddress, MHIP_ERUNTIME if that fails);
+ * no call allocates or frees.  All calls on one GPU share the array: calls that overlap in time on one GPU
+ * (different streams, different threads) race on it and must be serialised by the caller.  Arguments,
+ * results and error codes are otherwise those of mhip_attn_bwd_block.
+ */
+int mhip_attn_bwd_block_noalloc(const void* dout, const void* q, const void* k, const void* v,
+                                const void* out, const float* lse,
+                                void* dq, void* dk, void* dv, float* dq_acc,
+                                int B, int Sq, int Sc, int Hq, int Hkv, int D,
+                                int64_t q_sb, int64_t q_ss, int64_t q_sh,     /* q, out, dout, dq */
+                                int64_t k_sb, int64_t k_ss, int64_t k_sh,     /* k, v            */
+                                int64_t dk_sb, int64_t dk_ss, int64_t dk_sh,  /* dk, dv          */
+                                float softmax_scale, int mask, int deterministic, void* stream);
 
 /*
  * LSE-rescale merge.  Replaces the TorchScript `_update_out_and_lse`

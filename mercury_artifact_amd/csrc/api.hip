@@ -24,6 +24,8 @@ extern "C" const char* mhip_error_string(int code) {
     case MHIP_EALIGN: return "pointer or stride not aligned to 16 bytes";
     case MHIP_ELAUNCH: return "kernel launch failed";
     case MHIP_EUNSUPPORTED: return "feature not implemented";
+    case MHIP_ETOOLARGE: return "problem exceeds the built-in scratch of the no-allocation entry point (B * Hq * Sq <= 1048576)";
+    case MHIP_ERUNTIME: return "HIP runtime query failed (current device or symbol address)";
     default: return "unknown error code";
   }
 }

@@ -23,6 +23,8 @@
 // accumulator registers hold.
 #include "mhip_common.hpp"
 
+#include <atomic>
+
 namespace mhip {
 namespace {
 
@@ -532,22 +534,49 @@ extern "C" int64_t mhip_attn_bwd_workspace_bytes(int B, int Sq, int Sc, int Hq, 
   return (int64_t)B * Hq * Sq * 8 + 32;     // delta and lse2, (B, Hq, Sq) fp32 each
 }
 
-extern "C" int mhip_attn_bwd_block(const void* dout, const void* q, const void* k, const void* v,
-                                   const void* out, const float* lse,
-                                   void* dq, void* dk, void* dv, float* dq_acc,
-                                   int B, int Sq, int Sc, int Hq, int Hkv, int D,
-                                   int64_t q_sb, int64_t q_ss, int64_t q_sh,
-                                   int64_t k_sb, int64_t k_ss, int64_t k_sh,
-                                   int64_t dk_sb, int64_t dk_ss, int64_t dk_sh,
-                                   float softmax_scale, int mask, int deterministic,
-                                   void* workspace, void* stream) {
-  (void)deterministic;   // there are no atomics: every run is deterministic
+// Scratch of the entry point that allocates nothing: delta and lse2 of up to kScratchRows (batch, head, row)
+// triples.  Every GPU the library runs on holds its own copy until the process ends.
+constexpr int64_t kScratchRows = int64_t(1) << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchRows * 8 + 32];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device.  In host code the array's name is only a handle for
+// the runtime: the address a kernel can use comes from hipGetSymbolAddress, once per device.
+int scratch_address(void** ptr) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return MHIP_ERUNTIME;
+  void* cached = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (cached == nullptr) {
+    void* fresh = nullptr;
+    if (hipGetSymbolAddress(&fresh, HIP_SYMBOL(scratch)) != hipSuccess || fresh == nullptr) {
+      (void)hipGetLastError();
+      return MHIP_ERUNTIME;
+    }
+    g_scratch_ptr[dev].store(fresh, std::memory_order_release);   // every thread would store the same address
+    cached = fresh;
+  }
+  *ptr = cached;
+  return MHIP_OK;
+}
+
+// own_scratch: take the workspace from `scratch` (resolved after the arguments have been checked)
+int bwd_block(const void* dout, const void* q, const void* k, const void* v,
+              const void* out, const float* lse,
+              void* dq, void* dk, void* dv, float* dq_acc,
+              int B, int Sq, int Sc, int Hq, int Hkv, int D,
+              int64_t q_sb, int64_t q_ss, int64_t q_sh,
+              int64_t k_sb, int64_t k_ss, int64_t k_sh,
+              int64_t dk_sb, int64_t dk_ss, int64_t dk_sh,
+              float softmax_scale, int mask, void* workspace, bool own_scratch, hipStream_t st) {
   if (B < 0 || Sq < 0 || Sc < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return MHIP_EINVAL;
   if (!(softmax_scale > 0.f) || !(softmax_scale < INFINITY)) return MHIP_EINVAL;
   if (mask != MHIP_MASK_NONE && mask != MHIP_MASK_CAUSAL) return MHIP_EINVAL;
   if (D != kD) return MHIP_EHEADDIM;
   if (B == 0) return MHIP_OK;
-  if (Sq > 0 && (!dout || !q || !out || !lse || !dq || !workspace)) return MHIP_EINVAL;
+  if (Sq > 0 && (!dout || !q || !out || !lse || !dq || (!workspace && !own_scratch))) return MHIP_EINVAL;
   if (Sc > 0 && (!k || !v || !dk || !dv)) return MHIP_EINVAL;
   const void* ptrs[] = {dout, q, k, v, out, dq, dk, dv, workspace, dq_acc};
   for (const void* ptr : ptrs)
@@ -559,7 +588,11 @@ extern "C" int mhip_attn_bwd_block(const void* dout, const void* q, const void* 
   const int64_t q_span = ((int64_t)Sq * q_ss + (int64_t)Hq * q_sh) * 2;
   const int64_t k_span = (int64_t)Sc * k_ss * 2;
   if (q_span >= (int64_t(1) << 31) || k_span >= (int64_t(1) << 31)) return MHIP_EUNSUPPORTED;
-  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (own_scratch && Sq > 0) {
+    if ((int64_t)B * Hq * Sq > kScratchRows) return MHIP_ETOOLARGE;
+    const int rc = scratch_address(&workspace);
+    if (rc != MHIP_OK) return rc;
+  }
 
   BwdParams p;
   p.q = static_cast<const uint16_t*>(q); p.k = static_cast<const uint16_t*>(k);
@@ -599,4 +632,35 @@ extern "C" int mhip_attn_bwd_block(const void* dout, const void* q, const void* 
     else hipLaunchKernelGGL((bwd_main<false, false>), dim3(p.per_xcd * 8), dim3(256), 0, st, p);
   }
   return launch_status();
+}
+}  // namespace
+
+extern "C" int mhip_attn_bwd_block(const void* dout, const void* q, const void* k, const void* v,
+                                   const void* out, const float* lse,
+                                   void* dq, void* dk, void* dv, float* dq_acc,
+                                   int B, int Sq, int Sc, int Hq, int Hkv, int D,
+                                   int64_t q_sb, int64_t q_ss, int64_t q_sh,
+                                   int64_t k_sb, int64_t k_ss, int64_t k_sh,
+                                   int64_t dk_sb, int64_t dk_ss, int64_t dk_sh,
+                                   float softmax_scale, int mask, int deterministic,
+                                   void* workspace, void* stream) {
+  (void)deterministic;   // there are no atomics: every run is deterministic
+  return bwd_block(dout, q, k, v, out, lse, dq, dk, dv, dq_acc, B, Sq, Sc, Hq, Hkv, D, q_sb, q_ss, q_sh,
+                   k_sb, k_ss, k_sh, dk_sb, dk_ss, dk_sh, softmax_scale, mask, workspace, false,
+                   static_cast<hipStream_t>(stream));
+}
+
+extern "C" int mhip_attn_bwd_block_noalloc(const void* dout, const void* q, const void* k, const void* v,
+                                           const void* out, const float* lse,
+                                           void* dq, void* dk, void* dv, float* dq_acc,
+                                           int B, int Sq, int Sc, int Hq, int Hkv, int D,
+                                           int64_t q_sb, int64_t q_ss, int64_t q_sh,
+                                           int64_t k_sb, int64_t k_ss, int64_t k_sh,
+                                           int64_t dk_sb, int64_t dk_ss, int64_t dk_sh,
+                                           float softmax_scale, int mask, int deterministic, void* stream) {
+  (void)deterministic;
+  // bwd_prepare overwrites the part of the scratch the two main kernels read, so nothing has to be cleared
+  return bwd_block(dout, q, k, v, out, lse, dq, dk, dv, dq_acc, B, Sq, Sc, Hq, Hkv, D, q_sb, q_ss, q_sh,
+                   k_sb, k_ss, k_sh, dk_sb, dk_ss, dk_sh, softmax_scale, mask, nullptr, true,
+                   static_cast<hipStream_t>(stream));
 }
