@@ -50,6 +50,39 @@ def cpu_baseline(sample_heads: int, B: int, Sq: int, D: int, W: int):
                       f"matmul/logsumexp + merge), {dt:.1f} s"}
 
 
+# One rank's forward step as Mercury's generator spells it (mercury/backend/pytorch/codegen.py:264-355, 442-523
+# for the template utils/flash_attn_dsl.py:127-180): every name but torch is resolved in the exec namespace.
+GENERATED_STEP_TEXT = '''
+def generated_ring_step(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False, window_size=(-1, -1),
+                        alibi_slopes=None, deterministic=False):
+    indices = one_dim_to_n_dim(RANK, (WORLD,))
+    _out = None
+    _lse = None
+    for ring_idx in range(WORLD):
+        if ring_idx == 0:
+            _kv = kv[:, :, :, :, :].contiguous()
+            comm = SendRecv()
+        else:
+            comm.wait()
+            _kv = _next_kv
+        if ring_idx + 1 != WORLD:
+            send_to = n_dim_to_one_dim(shift_tuple_element(indices, 0, 1, WORLD), (WORLD,))
+            recv_from = n_dim_to_one_dim(shift_tuple_element(indices, 0, -1, WORLD), (WORLD,))
+            _next_kv = comm.send_recv(send_to, recv_from, _kv)
+            comm.commit()
+        params = get_default_args(_flash_attn_forward).copy()
+        params.update({"q": q, "k": _kv[0], "v": _kv[1], "dropout_p": dropout_p, "softmax_scale": softmax_scale,
+                       "causal": causal, "alibi_slopes": alibi_slopes, "return_softmax": True and dropout_p > 0,
+                       "window_size_left": window_size[0], "window_size_right": window_size[1]})
+        outputs = _flash_attn_forward(**params)
+        assert len(outputs) == 4
+        block_out, block_lse, _, _ = outputs
+        _out, _lse = update_out_and_lse(_out, _lse, block_out, block_lse)
+    o[:, :, :, :] = _out.to(q.dtype)
+    lse[:, :, :] = _lse.squeeze(dim=-1).transpose(1, 2)
+'''
+
+
 def other_kernels(torch, M, dev):
     """Block kernels of the other configurations at their per-rank shapes, HIP events over 10 launches each
     (reported next to the headline, not part of it)."""
@@ -243,8 +276,31 @@ def main() -> int:
     merge_ms = sum(e0.elapsed_time(e1) for e0, e1 in real_merges) / max(len(real_merges), 1)
     merge_gbs = merge_bytes / (merge_ms * 1e-3) / 1e9
 
-    # the same step replayed as one HIP graph (one launch instead of ~25; identical kernels and results)
+    # the drop-in boundary itself: a step function spelled the way the generator spells it (bare names resolved in
+    # the exec namespace, update_out_and_lse per chunk, the two epilogue stores), run unchanged in
+    # namespace(lazy_merge=True), where the merges of the step are recorded and folded once by the epilogue
     FI.attn_fwd_block, MG.merge_into, RG.merge_many = real_fwd, real_merge, real_many
+    drop_in_ms = {}
+    for lazy in (False, True):
+        ring_box = {}
+        ns = {"torch": torch, "WORLD": W, "RANK": rank, "SendRecv": lambda: ring_box["ring"]}
+        ns.update(M.namespace(lazy_merge=lazy))
+        exec(GENERATED_STEP_TEXT, ns)
+
+        def drop_in_step():
+            ring_box["ring"] = M.LocalRing((W,), rank, kvs)
+            ns["generated_ring_step"](q, kvs[rank], o, lse, scale)
+
+        for _ in range(2):
+            drop_in_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            drop_in_step()
+        torch.cuda.synchronize()
+        drop_in_ms[lazy] = (time.perf_counter() - t0) / args.steps * 1e3
+
+    # the same step replayed as one HIP graph (one launch instead of ~25; identical kernels and results)
     graph_ms, graph_same = None, None
     try:
         graphed = M.GraphedStep(step)
@@ -303,6 +359,9 @@ def main() -> int:
                                "of 4096 (single ring, rank 0), 8 block forwards + one fold of the 8 block results",
                    "flops_per_step": flops_per_step, "pct_of_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
                    "literal_merge_chain_ms_per_step": round(unfused_ms, 4),
+                   "generated_text_ms_per_step": round(drop_in_ms[False], 4),
+                   "generated_text_lazy_namespace_ms_per_step": round(drop_in_ms[True], 4),
+                   "generated_text_lazy_namespace_tflops": round(flops_per_step / drop_in_ms[True] / 1e9, 1),
                    "hip_graph_ms_per_step": graph_ms, "hip_graph_bit_identical": graph_same,
                    "device": props.gcnArchName, "cus": props.multi_processor_count,
                    "d2d_copy_gbs": round(copy_gbs, 1)},

@@ -139,7 +139,7 @@ int mhip_lse_merge(const float* acc_out, const float* acc_lse,
  *   final_out = bf16(sum_i exp(lse_i - L) * out_i),  final_lse = L,
  * which is what the chain computes (the fold is associative) without moving the fp32 accumulator through
  * memory N - 1 times.  block_outs / block_lses / bo_sb / s_begin are HOST arrays of n entries
- * (1 <= n <= 16; s_begin may be NULL = all zero).  Block i covers the sequence rows s >= s_begin[i]
+ * (1 <= n <= 64; s_begin may be NULL = all zero).  Block i covers the sequence rows s >= s_begin[i]
  * (rows before count as lse = -inf: the "second half of the Q rows" steps of a zigzag schedule):
  * block_outs[i] bf16 (B, Sq - s_begin[i], Hq, D) addressed with the element strides bo_sb[i], bo_ss, bo_sh
  * (multiples of 8, 16-byte aligned base, D contiguous), block_lses[i] fp32 (B, Hq, Sq - s_begin[i])

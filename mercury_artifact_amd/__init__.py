@@ -11,6 +11,7 @@ from . import _native
 from .flash_attn_interface import (_flash_attn_backward, _flash_attn_forward, attn_bwd_block,
                                    attn_fwd_block)
 from .graph import GraphedStep
+from .lazy import LazyLse, LazyOut, update_out_and_lse_lazy
 from .merge import (LocalGroup, _update_out_and_lse, add_collective, flash_reduce, get_default_args,
                     grad_accumulate, merge_into, merge_many, pack_block, unpack_into, update_out_and_lse,
                     update_out_and_lse_collective)
@@ -25,14 +26,19 @@ from .schedule import (LocalRing, double_ring_order, get_src_dst_ranks, n_dim_to
 __version__ = "0.1.0"
 
 
-def namespace() -> dict:
+def namespace(lazy_merge: bool = False) -> dict:
     """Names to place in the dict generated ring code is ``exec``-ed in (the reference fills it with
-    ``from utils.flash_attn_dsl import *`` and ``from mercury.backend import *``)."""
+    ``from utils.flash_attn_dsl import *`` and ``from mercury.backend import *``).
+
+    ``lazy_merge=True`` binds ``update_out_and_lse`` to the recording variant of ``mercury_artifact_amd.lazy``:
+    unchanged generated code then folds all block results of a step in one pass when its epilogue runs,
+    instead of moving the fp32 accumulator once per chunk (same results to fp32 rounding; anything the lazy
+    handles are not asked by the generated epilogue falls back to the literal chain)."""
     return {
         "_flash_attn_forward": _flash_attn_forward,
         "_flash_attn_backward": _flash_attn_backward,
         "get_default_args": get_default_args,
-        "update_out_and_lse": update_out_and_lse,
+        "update_out_and_lse": update_out_and_lse_lazy if lazy_merge else update_out_and_lse,
         "_update_out_and_lse": _update_out_and_lse,
         "flash_reduce": flash_reduce,
         "merge_many": merge_many,

@@ -471,7 +471,10 @@ __global__ __launch_bounds__(256) void unpack_kernel(const float* __restrict__ b
 // (0, -inf).  A block may cover only the rows s >= s_begin[i] of the sequence dimension (the zigzag
 // schedule's "second half of the Q rows" steps); the rows before count as lse = -inf.
 // One row = D/8 lanes x 8 contiguous head-dim values (16 bytes of bf16) per thread.
-constexpr int kMaxBlocks = 16;
+// More than kGroup blocks are folded in groups of kGroup with the running (maximum, sum, weighted output) carried
+// in registers, the online-softmax way, still in one pass over every block.
+constexpr int kMaxBlocks = 64;
+constexpr int kGroup = 16;
 struct MergeManyParams {
   const uint16_t* out[kMaxBlocks];
   const float* lse[kMaxBlocks];
@@ -483,10 +486,11 @@ struct MergeManyParams {
   int64_t bo_ss, bo_sh;
 };
 
-template <int LPR, int N>          // N = 0: run-time block count
+template <int LPR, int N>          // N = 0: run-time block count, folded in groups of kGroup
 __global__ __launch_bounds__(256) void lse_merge_many_kernel(const MergeManyParams p) {
   constexpr int D = LPR * 8;
   constexpr int kRowsPerPass = 256 / LPR;
+  constexpr int G = N > 0 ? N : kGroup;
   const int n = N > 0 ? N : p.n;
   const int64_t row = (int64_t)blockIdx.x * kRowsPerPass + threadIdx.x / LPR;
   if (row >= p.rows) return;
@@ -496,30 +500,38 @@ __global__ __launch_bounds__(256) void lse_merge_many_kernel(const MergeManyPara
   const uint32_t s = bs % (uint32_t)p.Sq;
   const uint32_t b = bs / (uint32_t)p.Sq;
   const int64_t l_off = ((int64_t)b * p.Hq + h) * p.Sq + s;
-  u32x4 blk[N > 0 ? N : kMaxBlocks];
-  float l[N > 0 ? N : kMaxBlocks];
+  float m = -INFINITY;             // maximum of the lse folded so far
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  float sum = 0.f;                 // both relative to m
+  for (int g0 = 0; g0 < n; g0 += G) {
+    u32x4 blk[G];
+    float l[G];
 #pragma unroll
-  for (int i = 0; i < (N > 0 ? N : kMaxBlocks); ++i) {
-    if (i < n) {
-      const int sb = p.s_begin[i];
+    for (int i = 0; i < G; ++i) {
       l[i] = -INFINITY;
       blk[i] = u32x4{0u, 0u, 0u, 0u};
-      if ((int)s >= sb) {
-        const int64_t o_off = b * p.bo_sb[i] + (int64_t)(s - sb) * p.bo_ss + h * p.bo_sh + col;
-        blk[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.out[i] + o_off));
-        l[i] = p.lse[i][((int64_t)b * p.Hq + h) * (p.Sq - sb) + (s - sb)];
+      if (g0 + i < n) {
+        const int sb = p.s_begin[g0 + i];
+        if ((int)s >= sb) {
+          const int64_t o_off = b * p.bo_sb[g0 + i] + (int64_t)(s - sb) * p.bo_ss + h * p.bo_sh + col;
+          blk[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.out[g0 + i] + o_off));
+          l[i] = p.lse[g0 + i][((int64_t)b * p.Hq + h) * (p.Sq - sb) + (s - sb)];
+        }
       }
     }
-  }
-  float m = -INFINITY;
+    float m_new = m;
 #pragma unroll
-  for (int i = 0; i < (N > 0 ? N : kMaxBlocks); ++i)
-    if (i < n) m = fmaxf(m, l[i]);
-  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  float sum = 0.f;
+    for (int i = 0; i < G; ++i) m_new = fmaxf(m_new, l[i]);
+    if (N == 0 && g0 > 0) {
+      // what was folded before this group moves to the new maximum (exp(-inf - x) = 0 handles an empty past)
+      const float carry = (m_new == -INFINITY) ? 0.f : __expf(m - m_new);
+      sum *= carry;
 #pragma unroll
-  for (int i = 0; i < (N > 0 ? N : kMaxBlocks); ++i) {
-    if (i < n) {
+      for (int j = 0; j < 8; ++j) acc[j] *= carry;
+    }
+    m = m_new;
+#pragma unroll
+    for (int i = 0; i < G; ++i) {
       const float w = (m == -INFINITY) ? 0.f : __expf(l[i] - m);
       sum += w;
 #pragma unroll

@@ -83,7 +83,7 @@ def merge_into(acc_out: Optional[torch.Tensor], acc_lse: Optional[torch.Tensor],
     N.check(code, "mhip_lse_merge")
 
 
-MAX_MERGE_MANY = 16
+MAX_MERGE_MANY = 64
 
 
 def merge_many(block_outs: Sequence[torch.Tensor], block_lses: Sequence[torch.Tensor],

@@ -19,6 +19,7 @@ sequence: ``update_out_and_lse`` per chunk, then ``o[...] = _out.to(o.dtype)``,
 """
 from __future__ import annotations
 
+import warnings
 from typing import Optional
 
 import torch
@@ -102,6 +103,10 @@ def _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, 
     n_blocks = len(steps) * ring_divide
     defer = (deferred_merge and n_blocks <= MAX_MERGE_MANY and o.dtype == torch.bfloat16
              and o.is_contiguous() and lse.is_contiguous())
+    if deferred_merge and not defer:
+        warnings.warn(f"ring step of {n_blocks} blocks into a {o.dtype} output: the one-pass fold takes at most "
+                      f"{MAX_MERGE_MANY} blocks and writes contiguous bfloat16, so this step merges block by block "
+                      "(same result, one pass over the fp32 accumulator per block)", RuntimeWarning, stacklevel=3)
     done = 0
     for part in range(ring_divide):
         rows = slice(part * sub, (part + 1) * sub)

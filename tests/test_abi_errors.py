@@ -79,7 +79,7 @@ def test_elementwise_rejects(lib):
     def many(outs=two, lses=two, sb=sb2, begin=None, n=2, fo=P, fl=P, D=128, st=(128 * 4, 128), B=1):
         return lib.mhip_lse_merge_many(outs, lses, sb, begin, n, fo, fl, B, 8, 4, D, *st, None)
 
-    assert many(n=0) == EINVAL and many(n=17) == EINVAL
+    assert many(n=0) == EINVAL and many(n=65) == EINVAL
     assert many(fo=None) == EINVAL and many(outs=None) == EINVAL and many(sb=None) == EINVAL
     assert many(outs=(ctypes.c_void_p * 2)(P, None)) == EINVAL
     assert many(begin=(ctypes.c_int * 2)(0, 9)) == EINVAL and many(begin=(ctypes.c_int * 2)(-1, 0)) == EINVAL

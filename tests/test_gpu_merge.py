@@ -218,7 +218,7 @@ def test_add_collective_sums_the_group():
         M.add_collective(mine, "reduce", M.LocalGroup(peers, rank=0))
 
 
-@pytest.mark.parametrize("n", [1, 2, 3, 8, 16])
+@pytest.mark.parametrize("n", [1, 2, 3, 8, 16, 17, 32, 45, 64])
 @pytest.mark.parametrize("B,Sq,H,D", [(2, 37, 3, 128), (1, 64, 4, 64), (1, 9, 2, 256)])
 def test_merge_many_matches_the_chain(n, B, Sq, H, D):
     """One fold of all block results against the chain of reference merges in fp64 followed by the
@@ -268,7 +268,7 @@ def test_merge_many_strided_blocks_and_errors():
     assert ((fo.float().cpu() - ro.float()).abs() - (1e-3 + 2 ** -8 * ro.float().abs())).max().item() <= 0
     assert torch.allclose(fl.cpu(), rl.float(), atol=1e-5, rtol=1e-5)
     with pytest.raises(RuntimeError):
-        M.merge_many(outs * 5, lses * 5, fo, fl)             # 20 blocks
+        M.merge_many(outs * 17, lses * 17, fo, fl)           # 68 blocks: one fold takes at most 64
     with pytest.raises(RuntimeError):
         M.merge_many(outs, lses[:-1], fo, fl)
     with pytest.raises(RuntimeError):

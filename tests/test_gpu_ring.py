@@ -57,7 +57,7 @@ def test_single_ring_reference_test_shape(rank, fused, deferred):
     assert torch.equal(qd, q_before) and torch.equal(dev_kvs[rank], kv_before)   # inputs untouched
 
 
-@pytest.mark.parametrize("divide,deferred", [(2, True), (4, True), (4, False)])
+@pytest.mark.parametrize("divide,deferred", [(2, True), (4, True), (4, False), (8, True), (16, True)])
 def test_single_ring_with_ring_divide(divide, deferred):
     """ring_divide = k (tests/test_ring_attn_codegen.py:102, benchmark/bench_attn.py:178): k * W block calls on
     sub-chunks in the order of the generated loops; the result is attention over all keys."""
@@ -96,6 +96,25 @@ def test_single_ring_with_ring_divide(divide, deferred):
     with pytest.raises(ValueError):
         M.flash_attn_pack_kv(qs[rank].cuda(), dev[rank], o, lse, scale, ring=M.LocalRing((W,), rank, dev),
                              ring_divide=7)
+
+
+def test_ring_divide_beyond_the_fold_limit_warns_and_merges_block_by_block():
+    """128 blocks (ring_divide 32 on 4 ranks) exceed what one fold takes: the driver says so and merges block by
+    block; the result is the same attention over all keys."""
+    import mercury_artifact_amd as M
+
+    B, S, H, D, W, rank, divide = 1, 2048, 2, 128, 4, 1, 32
+    q, k, v, qs, kvs = _inputs(B, S, H, H, D, W, seed=6)
+    scale = D ** -0.5
+    so, sl = O.single_pass_attention(qs[rank].float(), k.float(), v.float(), scale)
+    dev = [c.cuda() for c in kvs]
+    o = torch.empty(B, S // W, H, D, dtype=torch.bfloat16, device="cuda")
+    lse = torch.empty(B, H, S // W, dtype=torch.float32, device="cuda")
+    assert W * divide > M.merge.MAX_MERGE_MANY
+    with pytest.warns(RuntimeWarning, match="merges block by block"):
+        M.flash_attn_pack_kv(qs[rank].cuda(), dev[rank], o, lse, scale, ring=M.LocalRing((W,), rank, dev),
+                             ring_divide=divide)
+    _compare(o, lse, so, sl)
 
 
 def test_gqa_ring():
