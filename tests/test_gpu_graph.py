@@ -91,3 +91,50 @@ def test_search_harness_times_a_step():
     assert o.float().abs().max().item() > 0
     with pytest.raises(ImportError):
         SH.bench_program(object())          # the IR and its code generator are not part of this package
+
+
+@pytest.mark.parametrize("lazy", [False, True])
+def test_search_harness_bench_program_allocates_execs_and_times(lazy, capsys):
+    """bench_program end to end without the reference's package: a stand-in program (name + I/O buffers) and a
+    Lowering whose generator returns this repo's generated-style step text.  The harness must exec the text in a
+    namespace holding this package's operators, allocate zeros for written buffers and N(0,1) for the others in
+    the buffers' dtypes, run warm-up and timed calls, and report the program's buffer bytes."""
+    import types
+
+    import mercury_artifact_amd as M
+    from mercury_artifact_amd import search_harness as SH
+    from test_gpu_generated_style import SINGLE_RING_TEXT, _Dist
+
+    B, S, H, D, W, rank = 1, 256, 2, 128, 2, 1
+    Buf = types.SimpleNamespace
+    buffers = [Buf(tensor="q", shape=(B, S, H, D), dtype=torch.bfloat16, write=False),
+               Buf(tensor="kv", shape=(2, B, S, H, D), dtype=torch.bfloat16, write=False),
+               Buf(tensor="o", shape=(B, S, H, D), dtype=torch.bfloat16, write=True),
+               Buf(tensor="lse", shape=(B, H, S), dtype=torch.float32, write=True)]
+    program = Buf(name="ring_step", buffers=buffers, eliminated=False)
+    nbytes = sum(torch.empty(b.shape, dtype=b.dtype).numel() * torch.empty((), dtype=b.dtype).element_size() for b in buffers)
+    seen = {}
+
+    def generate(prog):
+        assert prog.eliminated                       # loops are eliminated before the text is generated
+        return SINGLE_RING_TEXT
+
+    low = SH.Lowering(eliminate_loops=lambda prog: setattr(prog, "eliminated", True), generate_code=generate,
+                      io_buffers=lambda prog: prog.buffers, buffer_bytes=lambda prog: nbytes)
+    other = [torch.randn(2, B, S, H, D, device="cuda").bfloat16() for _ in range(W)]
+
+    class Ring(M.LocalRing):                         # the hop of the generated loop, and a look at the arguments
+        def __init__(self):
+            super().__init__((W,), rank, other)
+
+        def send_recv(self, send_to, recv_from, tensor):
+            seen.setdefault("kv_dtype", tensor.dtype)
+            return super().send_recv(send_to, recv_from, tensor)
+
+    extra = {"torch": torch, "dist": _Dist(rank), "WORLD": W, "SendRecv": Ring}
+    ips, seconds, mem = SH.bench_program(program, extra, num_iter=3, kwargs={"softmax_scale": D ** -0.5},
+                                         log=True, lowering=low, lazy_merge=lazy)
+    assert ips > 0 and seconds > 0 and abs(ips * seconds - 3) < 1e-6 and mem == nbytes
+    assert seen["kv_dtype"] == torch.bfloat16
+    printed = capsys.readouterr().out
+    assert "def ring_step" in printed and "iter/s" in printed and "Memory cost" in printed
