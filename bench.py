@@ -83,6 +83,43 @@ def generated_ring_step(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False,
 '''
 
 
+def mfma_ceiling(torch, N, dev, cus):
+    """TFLOP/s and shader clock of a register-only loop of the bf16 MFMA (mhip_probe_mfma_ceiling), with constant
+    and with pseudo-random operands: what the power management of this box lets the matrix pipes sustain."""
+    sink = torch.empty(cus * 256, dtype=torch.float32, device=dev)
+    cyc = torch.zeros(1, dtype=torch.int64, device=dev)
+    out = {}
+    for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
+        iters = 40000                                  # x 32 MFMAs per wavefront: about 25 ms
+        for n in (iters // 20, iters):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            N.check(N.lib().mhip_probe_mfma_ceiling(N.ptr(sink), N.ptr(cyc), cus, n, rnd, N.stream_of(sink)), "probe")
+            e1.record()
+            torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1)
+        flops = cus * 4.0 * iters * 32 * 32768.0
+        out[name] = {"tflops": round(flops / ms / 1e9, 1), "clock_mhz": round(cyc.item() / ms / 1e3)}
+    return out
+
+
+def smi_snapshot():
+    """Socket power and clocks as `amd-smi metric --power --clock` prints them, read while the GPU is busy (the
+    caller has work queued).  Best effort: None when the tool is missing or refuses."""
+    import re
+    import subprocess
+    try:
+        res = subprocess.run(["amd-smi", "metric", "--power", "--clock"], stdout=subprocess.PIPE,
+                             stderr=subprocess.DEVNULL, text=True, timeout=20)
+    except (OSError, subprocess.SubprocessError):
+        return None
+    power = re.search(r"SOCKET_POWER:\s*([0-9.]+)\s*W", res.stdout)
+    clocks = [int(x) for x in re.findall(r"^\s*CLK:\s*([0-9]+)\s*MHz", res.stdout, flags=re.M)]
+    if not power and not clocks:
+        return None
+    return {"socket_power_w": float(power.group(1)) if power else None, "clk_mhz_first_entries": clocks[:9]}
+
+
 def other_kernels(torch, M, dev):
     """Block kernels of the other configurations at their per-rank shapes, HIP events over 10 launches each
     (reported next to the headline, not part of it)."""
@@ -158,6 +195,8 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--cpu-heads", type=int, default=32, help="heads in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--sustain", type=float, default=1.5,
+                    help="seconds of back-to-back steps for the `sustained` figure (0 = skip)")
     ap.add_argument("--no-variants", action="store_true",
                     help="skip the short timings of the causal, backward and fp8 block kernels")
     args = ap.parse_args()
@@ -247,6 +286,23 @@ def main() -> int:
 
     ms_per_step = dt / args.steps * 1e3
     flops_per_block = 4.0 * B * H * Sq * Sq * D
+    # the same step sustained: at least `--sustain` seconds of back-to-back steps (the 20-step window above is
+    # 40 ms; the clock the power management settles at shows only after a few hundred milliseconds)
+    sustained = None
+    if args.sustain > 0:
+        n_sus = max(int(args.sustain * 1e3 / ms_per_step) + 1, args.steps)
+        s0, s1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s0.record()
+        for _ in range(n_sus):
+            step()
+        s1.record()
+        smi = smi_snapshot()                      # read while the queued steps run
+        torch.cuda.synchronize()
+        sus_ms = s0.elapsed_time(s1) / n_sus
+        sustained = {"steps": n_sus, "seconds": round(sus_ms * n_sus / 1e3, 3), "ms_per_step": round(sus_ms, 4),
+                     "tflops": round(flops_per_block * W / sus_ms / 1e9, 1),
+                     "pct_of_bf16_mfma_peak": round(flops_per_block * W / sus_ms / 1e9 / PEAK_BF16_TFLOPS * 100, 2),
+                     "amd_smi_during_run": smi}
     flops_per_step = flops_per_block * W
     value = flops_per_step / (ms_per_step * 1e-3) / 1e12
 
@@ -377,6 +433,8 @@ def main() -> int:
                            "traffic": TRAFFIC_MERGE_BYTES, "avg_launch_ms": round(merge_ms, 5), "launches": len(real_merges),
                            "bytes_per_launch": merge_bytes},
     }
+    result["sustained"] = sustained
+    result["mfma_ceiling"] = mfma_ceiling(torch, M._native, dev, props.multi_processor_count)
     if variants is not None:
         result["other_kernels"] = variants
     if args.cpu_heads > 0:

@@ -205,6 +205,17 @@ int mhip_unpack(const float* buf, void* out, float* lse, int B, int Sq, int Hq, 
  */
 int mhip_grad_accumulate(const float* acc, const void* block, float* dst, int64_t n, void* stream);
 
+/*
+ * Measurement aid, no counterpart in the reference: a register-only loop of v_mfma_f32_32x32x16_bf16 (the
+ * instruction of the bf16 block kernels), `workgroups` workgroups of four wavefronts, `iters` x 32 MFMAs per
+ * wavefront, with operands that are constant (random_operands == 0) or pseudo-random bf16 values.  sink:
+ * workgroups * 256 floats, cycles: one 64-bit count of shader clocks spent in the loop by the first
+ * wavefront.  FLOP = workgroups * 4 * iters * 32 * 32768; bench.py times it to report the matrix-pipe ceiling
+ * the power management of the box allows, next to the attention kernels' figures.
+ */
+int mhip_probe_mfma_ceiling(float* sink, long long* cycles, int workgroups, int iters, int random_operands,
+                            void* stream);
+
 #ifdef __cplusplus
 }
 #endif

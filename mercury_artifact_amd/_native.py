@@ -37,6 +37,7 @@ _SIGNATURES = {
     "mhip_unpack": (c_int, [_P] * 3 + [_I] * 4 + [_P]),
     "mhip_grad_accumulate": (c_int, [_P] * 3 + [_L, _P]),
     "mhip_quantize_e4m3": (c_int, [_P, _I, _L, _P, _P, _P, _P]),
+    "mhip_probe_mfma_ceiling": (c_int, [_P, _P, _I, _I, _I, _P]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 

@@ -160,3 +160,41 @@ def test_bwd_full_size_chunk_properties():
     _check_grad("dq", dq[:, :, heads], rdq)
     _check_grad("dk", dkv[0][:, :, heads], rdk)
     _check_grad("dv", dkv[1][:, :, heads], rdv)
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_bwd_ring_full_size(fused):
+    """The backward configuration at full size (B1 H32 D128, Q 4096 x 8 KV chunks of 4096): the merged out / LSE
+    of the forward ring step feed the backward ring step; dQ accumulated in fp32 over the 8 chunks (inside the
+    kernel, or by the literal torch.add sequence) and two chunks' dK / dV are compared on three heads with the
+    oracle's ring backward from the same out / LSE."""
+    import mercury_artifact_amd as M
+
+    B, Sq, H, D, W, rank = 1, 4096, 32, 128, 8, 5
+    g = torch.Generator().manual_seed(9)
+    q = torch.randn(B, Sq, H, D, generator=g).bfloat16()
+    kvs = [torch.randn(2, B, Sq, H, D, generator=g).bfloat16() for _ in range(W)]
+    dout = torch.randn(B, Sq, H, D, generator=g).bfloat16()
+    scale = D ** -0.5
+    dev = [c.cuda() for c in kvs]
+    qd, dd = q.cuda(), dout.cuda()
+    o = torch.empty_like(qd)
+    lse = torch.empty(B, H, Sq, dtype=torch.float32, device="cuda")
+    M.flash_attn_pack_kv(qd, dev[rank], o, lse, scale, ring=M.LocalRing((W,), rank, dev))
+    dq = torch.empty_like(qd)
+    dkv = torch.empty_like(dev[rank])
+    got = {}
+    print(f"full-size backward ring, fused_accumulate={fused}", flush=True)
+    M.flash_attn_backward(qd, dev[rank], o, lse, dd, dq, dkv, scale, ring=M.LocalRing((W,), rank, dev),
+                          dkv_chunks=got, fused_accumulate=fused)
+    torch.cuda.synchronize()
+    assert sorted(got) == list(range(W))
+    heads = [0, 13, 31]
+    order = O.single_ring_order(rank, W)
+    rdq, rdkv = O.ring_backward(q[:, :, heads].float(), [c[:, :, :, heads].float() for c in kvs], order,
+                                o[:, :, heads].float().cpu(), lse[:, heads].cpu(), dout[:, :, heads].float(), scale)
+    _check_grad("dq", dq[:, :, heads], rdq)
+    for c in (order[0], order[-1]):
+        _check_grad(f"dk[{c}]", got[c][0][:, :, heads], rdkv[c][0])
+        _check_grad(f"dv[{c}]", got[c][1][:, :, heads], rdkv[c][1])
+    assert torch.equal(dkv.float(), got[rank])          # the rank's own chunk is what dkv receives
