@@ -184,7 +184,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
   constexpr float kSlack = 14.f;          // rows whose maximum exceeds the reference by 2^kSlack move it
   const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   f32x16 s[2];               // S^T tile: 64 keys x 32 q rows per wave
-  bf16x8 pf[4];              // P^T of the current tile as bf16 B operands
+  u32x4 pw[4];               // P^T of the current tile as packed bf16 B operands, one per k-step
 
   auto qk = [&](int stage) {
     const unsigned char* ks = smem + stage * kTileBytes;
@@ -205,7 +205,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
 #pragma unroll
       for (int db = 0; db < 4; ++db) {
         const bf16x8 vf = read_v(vs, db, kstep);
-        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kstep], o_acc[db], 0, 0, 0);
+        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, __builtin_bit_cast(bf16x8, pw[kstep]), o_acc[db], 0, 0, 0);
       }
     }
   };
@@ -227,25 +227,26 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
         }
     }
   };
-  // exponentials of the tile, P^T as bf16 B operands (k-step (mb, j2) takes accumulator registers
-  // 8 j2 .. 8 j2 + 7) and this lane's sum of them; s stays intact
+  // Exponentials of the tile in 16 pairs: pair idx covers accumulator registers 2 idx, 2 idx + 1 (counted over
+  // both 32-key blocks) and gives one dword of the packed P^T operand of k-step idx / 4.  s stays intact.
+  // The first kEarlyPairs pairs are computed inside the matrix phase, between the O^T MFMAs: measured with
+  // cycle counters the vector phase is the longer of the two (1314 against 1265 ticks per 64-key tile), and
+  // two pairs moved over make the step 3 % faster (four and more slow the matrix phase down by as much as
+  // they shorten the other).  A pair may overwrite the P^T operand of k-step ks only after the last MFMA of
+  // that k-step has been issued.
   float rs = 0.f;
+  auto sm_pair = [&](int idx) {
+    const int mb = idx >> 3, r = (idx & 7) * 2;
+    float x0 = fast_exp2(__builtin_fmaf(s[mb][r], p.scale_log2, nmsc));
+    float x1 = fast_exp2(__builtin_fmaf(s[mb][r + 1], p.scale_log2, nmsc));
+    if (idx == 0) rs = x0 + x1; else rs += x0 + x1;
+    uint32_t w = pack_bf16(x0, x1);
+    asm volatile("" : "+v"(w), "+v"(rs));          // keeps the pair where it is written
+    pw[idx >> 2][idx & 3] = w;
+  };
   auto sm_exps = [&]() {
-    rs = 0.f;
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-      for (int j2 = 0; j2 < 2; ++j2) {
-        u32x4 w;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float x0 = fast_exp2(__builtin_fmaf(s[mb][8 * j2 + 2 * e], p.scale_log2, nmsc));
-          const float x1 = fast_exp2(__builtin_fmaf(s[mb][8 * j2 + 2 * e + 1], p.scale_log2, nmsc));
-          w[e] = pack_bf16(x0, x1);
-          rs += x0 + x1;
-        }
-        pf[mb * 2 + j2] = __builtin_bit_cast(bf16x8, w);
-      }
+    for (int idx = 0; idx < 16; ++idx) sm_pair(idx);
   };
   // Move the reference of the rows whose scores outgrew it (first tile: set it to the row maximum) and
   // rescale O and the running sum accordingly.
@@ -269,8 +270,19 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     m_ref = move ? mx : m_ref;
     nmsc = -m_ref * p.scale_log2;
   };
+#ifndef MHIP_FWD_EARLY_PAIRS
+#define MHIP_FWD_EARLY_PAIRS 2
+#endif
+  constexpr int kEarlyPairs = MHIP_FWD_EARLY_PAIRS;
+  // slot of the matrix phase after which early pair idx runs: k-step idx / 4 of the tile before is read by
+  // slots 16 + 4 (idx / 4) .. + 3, and the pairs are spread two slots apart behind that
+#ifndef MHIP_FWD_EARLY_STEP
+#define MHIP_FWD_EARLY_STEP 2
+#endif
+  auto early_slot = [](int idx) { return idx < 4 ? 20 + MHIP_FWD_EARLY_STEP * idx : 28 + (idx - 4); };
   auto sm_tile = [&]() {
-    sm_exps();
+#pragma unroll
+    for (int idx = kEarlyPairs; idx < 16; ++idx) sm_pair(idx);
     if (__builtin_amdgcn_ballot_w64(!(rs < kTrigger)) != 0) {
       sm_fix(false);
       sm_exps();
@@ -303,11 +315,14 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
         s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag[i % kFragDepth], qf[kk], kk == 0 ? zero : s[mb], 0, 0, 0);
       } else {
         const int db = (i - 16) & 3, kstep = (i - 16) >> 2;
-        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag[i % kFragDepth], pf[kstep], o_acc[db], 0, 0, 0);
+        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag[i % kFragDepth], __builtin_bit_cast(bf16x8, pw[kstep]), o_acc[db], 0, 0, 0);
       }
       if (i + kFragDepth < 32) frag[i % kFragDepth] = read_frag(i + kFragDepth, ks, vs);
       // S^T(t_next) is complete after slot 15; its softmax starts here, in the shadow of the O^T MFMAs
       if (i == 16) sm_mask(t_next);
+#pragma unroll
+      for (int idx = 0; idx < kEarlyPairs; ++idx)
+        if (early_slot(idx) == i) sm_pair(idx);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
