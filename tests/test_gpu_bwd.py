@@ -198,3 +198,19 @@ def test_bwd_ring_full_size(fused):
         _check_grad(f"dk[{c}]", got[c][0][:, :, heads], rdkv[c][0])
         _check_grad(f"dv[{c}]", got[c][1][:, :, heads], rdkv[c][1])
     assert torch.equal(dkv.float(), got[rank])          # the rank's own chunk is what dkv receives
+
+
+def test_bwd_block_head_dim_64():
+    """Head dimension 64 through the backward (zero-padded operands, gradients of the padding dropped)."""
+    import mercury_artifact_amd as M
+
+    q, kv, dout, o16, lse, scale, (rdq, rdk, rdv) = _case(2, 160, 200, 4, 2, True, seed=12, D=64)
+    qd, kvd, dd, od, ld = q.cuda(), kv.cuda(), dout.cuda(), o16.cuda(), lse.cuda()
+    dq = torch.full_like(qd, float("nan")); dkv = torch.full_like(kvd, float("nan"))
+    acc = torch.full(qd.shape, 0.5, dtype=torch.float32, device="cuda")
+    M.attn_bwd_block(dd, qd, kvd[0], kvd[1], od, ld, dq, dkv[0], dkv[1], scale, causal=True, dq_acc=acc)
+    torch.cuda.synchronize()
+    _check_grad("dq", dq, rdq)
+    _check_grad("dk", dkv[0], rdk)
+    _check_grad("dv", dkv[1], rdv)
+    _check_grad("dq_acc", acc - 0.5, rdq)

@@ -167,8 +167,11 @@ def test_fwd_rejects_what_it_does_not_implement():
                               window_size_left=-1, window_size_right=-1, softcap=0.0, alibi_slopes=None,
                               return_softmax=False)
     with pytest.raises(RuntimeError):
-        M.attn_fwd_block(qd[..., :64].contiguous(), kvd[0][..., :64].contiguous(),
-                         kvd[1][..., :64].contiguous(), 0.1)      # head dim 64
+        M.attn_fwd_block(qd[..., :100].contiguous(), kvd[0][..., :100].contiguous(),
+                         kvd[1][..., :100].contiguous(), 0.1)     # head dim 100: not a multiple of 8
+    big = torch.zeros(1, 64, 2, 256, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError):
+        M.attn_fwd_block(big, big, big, 0.1)                      # head dim 256: beyond the kernels' 128
     with pytest.raises(RuntimeError):
         M.attn_fwd_block(qd.float(), kvd[0].float(), kvd[1].float(), 0.1)
     with pytest.raises(RuntimeError):
@@ -201,3 +204,44 @@ def test_fwd_chunks_merge_to_single_pass_full_size():
     heads = [0, 13, 31]
     ro, rl = O.block_attention(q[:, :, heads].float(), k[:, :, heads].float(), v[:, :, heads].float(), scale)
     _check(o[:, :, heads], lse[:, heads], ro, rl, "config1")
+
+
+@pytest.mark.parametrize("D,causal", [(64, False), (64, True), (32, False), (96, True)])
+def test_fwd_block_smaller_head_dims(D, causal):
+    """Head dimensions below 128 (multiples of 8) run through the same kernel on zero-padded operands."""
+    import mercury_artifact_amd as M
+
+    B, Sq, Sc, Hq, Hkv = 2, 200, 330, 4, 2
+    q, kv = _mk(B, Sq, Sc, Hq, Hkv, D=D, seed=31)
+    scale = D ** -0.5
+    ro, rl = O.block_attention(q.float(), kv[0].float(), kv[1].float(), scale, causal=causal)
+    out, lse = M.attn_fwd_block(q.cuda(), kv[0].cuda(), kv[1].cuda(), scale, causal=causal)
+    assert out.shape == (B, Sq, Hq, D) and out.is_contiguous()
+    _check(out, lse, ro, rl, f"D{D}")
+    into = torch.full((B, Sq, Hq, D), 7.0, dtype=torch.bfloat16, device="cuda")
+    o2, l2 = M.attn_fwd_block(q.cuda(), kv[0].cuda(), kv[1].cuda(), scale, causal=causal, out=into)
+    assert o2 is into and torch.equal(into, out) and torch.equal(l2, lse)
+
+
+def test_config0_through_the_gpu_path():
+    """BASELINE configuration 0 (the CPU plumbing case: B1 H4 D64, Q 1024 x 4 KV chunks of 256, N(0,1) from
+    torch.manual_seed(0), scale 1/8) through libmercury_hip.so: the inputs are rounded to bf16 (the block
+    operator takes no fp32, like the flash-attn operator it replaces) and every rank's ring step -- one fold,
+    the literal chain, and unchanged generated-style text in the lazy namespace -- is compared with single-pass
+    fp32 attention over all 1024 keys on the same rounded values."""
+    import mercury_artifact_amd as M
+
+    torch.manual_seed(0)
+    q, k, v = (torch.randn(1, 1024, 4, 64).bfloat16() for _ in range(3))
+    scale = 64 ** -0.5
+    chunks = [torch.stack([k[:, c * 256:(c + 1) * 256], v[:, c * 256:(c + 1) * 256]]) for c in range(4)]
+    ref_o, ref_l = O.single_pass_attention(q.float(), k.float(), v.float(), scale)
+    dev = [c.cuda() for c in chunks]
+    qd = q.cuda()
+    for rank in range(4):
+        for deferred in (True, False):
+            o = torch.empty_like(qd)
+            lse = torch.empty(1, 4, 1024, dtype=torch.float32, device="cuda")
+            M.flash_attn_pack_kv(qd, dev[rank], o, lse, scale, ring=M.LocalRing((4,), rank, dev),
+                                 deferred_merge=deferred, fused_epilogue=deferred)
+            _check(o, lse, ref_o, ref_l, f"config0 rank {rank} deferred={deferred}")
