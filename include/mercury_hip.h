@@ -73,16 +73,20 @@ int mhip_attn_fwd_block(const void* q, const void* k, const void* v, void* out, 
  * (B,Sc,Hkv,D) in bf16.  If dq_acc (fp32, contiguous (B,Sq,Hq,D)) is not NULL the block's
  * dq is ALSO added into it in fp32 -- the `reduce(op=torch.add, buffer=reduce_dq, ...)`
  * of utils/attn_bwd_dsl.py:117-122 folded into the kernel.  `workspace` must hold
- * mhip_attn_bwd_workspace_bytes(...) bytes of device memory.
+ * mhip_attn_bwd_workspace_bytes(...) bytes of device memory.  dq and out have element strides of their own:
+ * the call site allocates block_dq with torch.empty (contiguous, utils/attn_bwd_dsl.py:83) while q, out and
+ * dout are views of the step's buffers; q and dout, k and v, dk and dv share a stride triple each.
  */
 int64_t mhip_attn_bwd_workspace_bytes(int B, int Sq, int Sc, int Hq, int Hkv, int D);
 int mhip_attn_bwd_block(const void* dout, const void* q, const void* k, const void* v,
                         const void* out, const float* lse,
                         void* dq, void* dk, void* dv, float* dq_acc,
                         int B, int Sq, int Sc, int Hq, int Hkv, int D,
-                        int64_t q_sb, int64_t q_ss, int64_t q_sh,     /* q, out, dout, dq */
-                        int64_t k_sb, int64_t k_ss, int64_t k_sh,     /* k, v            */
-                        int64_t dk_sb, int64_t dk_ss, int64_t dk_sh,  /* dk, dv          */
+                        int64_t q_sb, int64_t q_ss, int64_t q_sh,     /* q, dout  */
+                        int64_t k_sb, int64_t k_ss, int64_t k_sh,     /* k, v     */
+                        int64_t dk_sb, int64_t dk_ss, int64_t dk_sh,  /* dk, dv   */
+                        int64_t dq_sb, int64_t dq_ss, int64_t dq_sh,  /* dq       */
+                        int64_t o_sb, int64_t o_ss, int64_t o_sh,     /* out      */
                         float softmax_scale, int mask, int deterministic,
                         void* workspace, void* stream);
 
@@ -101,9 +105,11 @@ int mhip_attn_bwd_block_noalloc(const void* dout, const void* q, const void* k, 
                                 const void* out, const float* lse,
                                 void* dq, void* dk, void* dv, float* dq_acc,
                                 int B, int Sq, int Sc, int Hq, int Hkv, int D,
-                                int64_t q_sb, int64_t q_ss, int64_t q_sh,     /* q, out, dout, dq */
-                                int64_t k_sb, int64_t k_ss, int64_t k_sh,     /* k, v            */
-                                int64_t dk_sb, int64_t dk_ss, int64_t dk_sh,  /* dk, dv          */
+                                int64_t q_sb, int64_t q_ss, int64_t q_sh,     /* q, dout  */
+                                int64_t k_sb, int64_t k_ss, int64_t k_sh,     /* k, v     */
+                                int64_t dk_sb, int64_t dk_ss, int64_t dk_sh,  /* dk, dv   */
+                                int64_t dq_sb, int64_t dq_ss, int64_t dq_sh,  /* dq       */
+                                int64_t o_sb, int64_t o_ss, int64_t o_sh,     /* out      */
                                 float softmax_scale, int mask, int deterministic, void* stream);
 
 /*

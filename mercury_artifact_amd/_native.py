@@ -27,8 +27,8 @@ _SIGNATURES = {
     "mhip_error_string": (ctypes.c_char_p, [_I]),
     "mhip_attn_fwd_block": (c_int, [_P] * 5 + [_I] * 6 + [_L] * 12 + [_F, _I, _I, _F, _F, _F, _P]),
     "mhip_attn_bwd_workspace_bytes": (c_int64, [_I] * 6),
-    "mhip_attn_bwd_block": (c_int, [_P] * 10 + [_I] * 6 + [_L] * 9 + [_F, _I, _I, _P, _P]),
-    "mhip_attn_bwd_block_noalloc": (c_int, [_P] * 10 + [_I] * 6 + [_L] * 9 + [_F, _I, _I, _P]),
+    "mhip_attn_bwd_block": (c_int, [_P] * 10 + [_I] * 6 + [_L] * 15 + [_F, _I, _I, _P, _P]),
+    "mhip_attn_bwd_block_noalloc": (c_int, [_P] * 10 + [_I] * 6 + [_L] * 15 + [_F, _I, _I, _P]),
     "mhip_lse_merge": (c_int, [_P] * 8 + [_I] * 4 + [_L] * 17 + [_P]),
     "mhip_lse_merge_many": (c_int, [_P, _P, _P, _P, _I, _P, _P] + [_I] * 4 + [_L] * 2 + [_P]),
     "mhip_flash_reduce": (c_int, [_P] * 3 + [_L, _I, _P]),

@@ -44,7 +44,7 @@ struct BwdParams {
   const float* lse2; const float* delta;   // both (B, Hq, Sq) fp32, written by bwd_prepare
   uint16_t* dq; uint16_t* dk; uint16_t* dv; float* dq_acc;
   int B, Sq, Sc, Hq, Hkv, group;
-  int64_t q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, dk_sb, dk_ss, dk_sh;
+  int64_t q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, dk_sb, dk_ss, dk_sh, dq_sb, dq_ss, dq_sh, o_sb, o_ss, o_sh;
   float scale, scale_log2;
   int n_tiles;      // stationary tiles per (batch, head)
   int total;
@@ -56,7 +56,8 @@ struct BwdParams {
 __global__ __launch_bounds__(256) void bwd_prepare(const uint16_t* __restrict__ dout, const uint16_t* __restrict__ out,
                                                    const float* __restrict__ lse, float* __restrict__ delta,
                                                    float* __restrict__ lse2, int B, int Sq, int Hq,
-                                                   int64_t sb, int64_t ss, int64_t sh) {
+                                                   int64_t sb, int64_t ss, int64_t sh,
+                                                   int64_t o_sb, int64_t o_ss, int64_t o_sh) {
   const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   const int64_t rows = (int64_t)B * Hq * Sq;
   const int c = threadIdx.x & 15;
@@ -68,7 +69,7 @@ __global__ __launch_bounds__(256) void bwd_prepare(const uint16_t* __restrict__ 
     const int b = (int)(bh / Hq);
     const int64_t off = b * sb + (int64_t)s * ss + h * sh + c * 8;
     const u32x4 a = *reinterpret_cast<const u32x4*>(dout + off);
-    const u32x4 o = *reinterpret_cast<const u32x4*>(out + off);
+    const u32x4 o = *reinterpret_cast<const u32x4*>(out + (b * o_sb + (int64_t)s * o_ss + h * o_sh + c * 8));
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc += bf16_lo(a[j]) * bf16_lo(o[j]) + bf16_hi(a[j]) * bf16_hi(o[j]);
   }
@@ -502,7 +503,7 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     }
   };
   if (DQ) {
-    write_out(acc1, p.scale, p.dq, p.q_sb, p.q_ss, p.q_sh, hs);
+    write_out(acc1, p.scale, p.dq, p.dq_sb, p.dq_ss, p.dq_sh, hs);
     if (p.dq_acc != nullptr && my_r < n_st) {
       // fp32 accumulator (B, Sq, Hq, D) contiguous; every element belongs to exactly one lane
       float* ap = p.dq_acc + (((int64_t)b * p.Sq + my_r) * p.Hq + hs) * kD;
@@ -570,6 +571,8 @@ int bwd_block(const void* dout, const void* q, const void* k, const void* v,
               int64_t q_sb, int64_t q_ss, int64_t q_sh,
               int64_t k_sb, int64_t k_ss, int64_t k_sh,
               int64_t dk_sb, int64_t dk_ss, int64_t dk_sh,
+              int64_t dq_sb, int64_t dq_ss, int64_t dq_sh,
+              int64_t o_sb, int64_t o_ss, int64_t o_sh,
               float softmax_scale, int mask, void* workspace, bool own_scratch, hipStream_t st) {
   if (B < 0 || Sq < 0 || Sc < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return MHIP_EINVAL;
   if (!(softmax_scale > 0.f) || !(softmax_scale < INFINITY)) return MHIP_EINVAL;
@@ -581,7 +584,8 @@ int bwd_block(const void* dout, const void* q, const void* k, const void* v,
   const void* ptrs[] = {dout, q, k, v, out, dq, dk, dv, workspace, dq_acc};
   for (const void* ptr : ptrs)
     if (ptr && !aligned16(ptr)) return MHIP_EALIGN;
-  const int64_t strides[] = {q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, dk_sb, dk_ss, dk_sh};
+  const int64_t strides[] = {q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, dk_sb, dk_ss, dk_sh, dq_sb, dq_ss, dq_sh,
+                             o_sb, o_ss, o_sh};
   for (int64_t s : strides)
     if (s < 0 || (s & 7)) return MHIP_EALIGN;
   // streamed tiles are fetched through 32-bit buffer offsets
@@ -606,6 +610,8 @@ int bwd_block(const void* dout, const void* q, const void* k, const void* v,
   p.q_sb = q_sb; p.q_ss = q_ss; p.q_sh = q_sh;
   p.k_sb = k_sb; p.k_ss = k_ss; p.k_sh = k_sh;
   p.dk_sb = dk_sb; p.dk_ss = dk_ss; p.dk_sh = dk_sh;
+  p.dq_sb = dq_sb; p.dq_ss = dq_ss; p.dq_sh = dq_sh;
+  p.o_sb = o_sb; p.o_ss = o_ss; p.o_sh = o_sh;
   p.scale = softmax_scale; p.scale_log2 = softmax_scale * kLog2e;
   const bool causal = mask == MHIP_MASK_CAUSAL;
 
@@ -613,7 +619,7 @@ int bwd_block(const void* dout, const void* q, const void* k, const void* v,
     const int64_t rows = (int64_t)B * Hq * Sq;
     hipLaunchKernelGGL(bwd_prepare, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
                        static_cast<const uint16_t*>(dout), static_cast<const uint16_t*>(out), lse,
-                       delta_buf, lse2_buf, B, Sq, Hq, q_sb, q_ss, q_sh);
+                       delta_buf, lse2_buf, B, Sq, Hq, q_sb, q_ss, q_sh, o_sb, o_ss, o_sh);
     // dQ: one workgroup per 128 query rows
     p.n_tiles = (Sq + kRowsPerWg - 1) / kRowsPerWg;
     p.total = B * Hq * p.n_tiles;
@@ -642,11 +648,14 @@ extern "C" int mhip_attn_bwd_block(const void* dout, const void* q, const void* 
                                    int64_t q_sb, int64_t q_ss, int64_t q_sh,
                                    int64_t k_sb, int64_t k_ss, int64_t k_sh,
                                    int64_t dk_sb, int64_t dk_ss, int64_t dk_sh,
+                                   int64_t dq_sb, int64_t dq_ss, int64_t dq_sh,
+                                   int64_t o_sb, int64_t o_ss, int64_t o_sh,
                                    float softmax_scale, int mask, int deterministic,
                                    void* workspace, void* stream) {
   (void)deterministic;   // there are no atomics: every run is deterministic
   return bwd_block(dout, q, k, v, out, lse, dq, dk, dv, dq_acc, B, Sq, Sc, Hq, Hkv, D, q_sb, q_ss, q_sh,
-                   k_sb, k_ss, k_sh, dk_sb, dk_ss, dk_sh, softmax_scale, mask, workspace, false,
+                   k_sb, k_ss, k_sh, dk_sb, dk_ss, dk_sh, dq_sb, dq_ss, dq_sh, o_sb, o_ss, o_sh, softmax_scale, mask,
+                   workspace, false,
                    static_cast<hipStream_t>(stream));
 }
 
@@ -657,10 +666,13 @@ extern "C" int mhip_attn_bwd_block_noalloc(const void* dout, const void* q, cons
                                            int64_t q_sb, int64_t q_ss, int64_t q_sh,
                                            int64_t k_sb, int64_t k_ss, int64_t k_sh,
                                            int64_t dk_sb, int64_t dk_ss, int64_t dk_sh,
+                                           int64_t dq_sb, int64_t dq_ss, int64_t dq_sh,
+                                           int64_t o_sb, int64_t o_ss, int64_t o_sh,
                                            float softmax_scale, int mask, int deterministic, void* stream) {
   (void)deterministic;
   // bwd_prepare overwrites the part of the scratch the two main kernels read, so nothing has to be cleared
   return bwd_block(dout, q, k, v, out, lse, dq, dk, dv, dq_acc, B, Sq, Sc, Hq, Hkv, D, q_sb, q_ss, q_sh,
-                   k_sb, k_ss, k_sh, dk_sb, dk_ss, dk_sh, softmax_scale, mask, nullptr, true,
+                   k_sb, k_ss, k_sh, dk_sb, dk_ss, dk_sh, dq_sb, dq_ss, dq_sh, o_sb, o_ss, o_sh, softmax_scale, mask,
+                   nullptr, true,
                    static_cast<hipStream_t>(stream));
 }

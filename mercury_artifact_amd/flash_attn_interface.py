@@ -193,13 +193,17 @@ def attn_bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_scale, c
                                or not dq_acc.is_contiguous()):
         raise RuntimeError("dq_acc must be a contiguous float32 tensor of q's shape")
 
-    # the C ABI takes one stride triple for (q, out, dout, dq), one for (k, v), one for (dk, dv)
+    # the C ABI takes one stride triple each for (q, dout), (k, v), (dk, dv), dq and out
     def same(*ts):
-        return all(t.stride() == ts[0].stride() and t.stride(-1) == 1 for t in ts)
-    qq, oo, dd, dq_w = (q, out, dout, dq) if same(q, out, dout, dq) else \
-        (q.contiguous(), out.contiguous(), dout.contiguous(), torch.empty_like(q, memory_format=torch.contiguous_format))
-    kk, vv = (k, v) if same(k, v) else (k.contiguous(), v.contiguous())
-    dk_w, dv_w = (dk, dv) if same(dk, dv) else \
+        return all(t.stride() == ts[0].stride() for t in ts)
+
+    def rows_ok(t):
+        return t.stride(-1) == 1 and all(st % 8 == 0 for st in t.stride()[:-1])
+    qq, dd = (q, dout) if same(q, dout) and rows_ok(q) else (q.contiguous(), dout.contiguous())
+    oo = out if rows_ok(out) else out.contiguous()
+    dq_w = dq if rows_ok(dq) else torch.empty_like(q, memory_format=torch.contiguous_format)
+    kk, vv = (k, v) if same(k, v) and rows_ok(k) else (k.contiguous(), v.contiguous())
+    dk_w, dv_w = (dk, dv) if same(dk, dv) and rows_ok(dk) else \
         (torch.empty_like(k, memory_format=torch.contiguous_format),
          torch.empty_like(v, memory_format=torch.contiguous_format))
     lib = N.lib()
@@ -210,7 +214,7 @@ def attn_bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_scale, c
             N.ptr(dd), N.ptr(qq), N.ptr(kk), N.ptr(vv), N.ptr(oo), N.ptr(softmax_lse),
             N.ptr(dq_w), N.ptr(dk_w), N.ptr(dv_w), N.ptr(dq_acc),
             B, Sq, Sc, Hq, Hkv, D,
-            *_strides3(qq), *_strides3(kk), *_strides3(dk_w),
+            *_strides3(qq), *_strides3(kk), *_strides3(dk_w), *_strides3(dq_w), *_strides3(oo),
             float(softmax_scale), N.MASK_CAUSAL if causal else N.MASK_NONE, int(bool(deterministic)),
             N.ptr(ws), N.stream_of(q))
     N.check(code, "mhip_attn_bwd_block")

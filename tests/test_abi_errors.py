@@ -51,7 +51,8 @@ def test_forward_rejects(lib):
 def test_backward_rejects(lib):
     def bwd(B=1, Sq=64, Sc=64, Hq=2, Hkv=2, D=128, scale=0.1, mask=0, dq=P, ws=P, strides=None, dq_acc=None):
         if strides is None:
-            strides = [Sq * Hq * D, Hq * D, D, Sc * Hkv * D, Hkv * D, D, Sc * Hkv * D, Hkv * D, D]
+            strides = [Sq * Hq * D, Hq * D, D, Sc * Hkv * D, Hkv * D, D, Sc * Hkv * D, Hkv * D, D,
+                       Sq * Hq * D, Hq * D, D, Sq * Hq * D, Hq * D, D]
         return lib.mhip_attn_bwd_block(P, P, P, P, P, P, dq, P, P, dq_acc, B, Sq, Sc, Hq, Hkv, D, *strides,
                                        scale, mask, 0, ws, None)
 
@@ -62,8 +63,10 @@ def test_backward_rejects(lib):
     assert bwd(dq=None) == EINVAL
     assert bwd(ws=None) == EINVAL
     assert bwd(dq=P + 4) == EALIGN
-    assert bwd(strides=[64 * 256, 257, 128, 64 * 256, 256, 128, 64 * 256, 256, 128]) == EALIGN
-    assert bwd(Sq=4096, strides=[1 << 33, 1 << 21, 128, 64 * 256, 256, 128, 64 * 256, 256, 128]) == EUNSUPPORTED
+    assert bwd(strides=[64 * 256, 257, 128, 64 * 256, 256, 128, 64 * 256, 256, 128] + [64 * 256, 256, 128] * 2) == EALIGN
+    assert bwd(strides=[64 * 256, 256, 128] * 3 + [64 * 256, 260, 128, 64 * 256, 256, 128]) == EALIGN     # dq rows
+    assert bwd(Sq=4096, strides=[1 << 33, 1 << 21, 128, 64 * 256, 256, 128, 64 * 256, 256, 128]
+               + [4096 * 256, 256, 128] * 2) == EUNSUPPORTED
     assert bwd(B=0) == OK
     assert lib.mhip_attn_bwd_workspace_bytes(2, 100, 64, 4, 2, 128) >= 2 * 2 * 4 * 100 * 4
 

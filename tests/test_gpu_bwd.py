@@ -48,6 +48,7 @@ BWD_SHAPES = [
     (1, 64, 700, 1, 1, False),       # few rows, many keys
     (1, 700, 64, 3, 1, False),       # many rows of three grouped heads, few keys
     (1, 1, 2, 1, 1, False),          # a single query row (with one key every gradient of q is exactly zero)
+    (2, 384, 384, 8, 4, True),       # causal with B*Hq and B*Hkv multiples of 8: the per-XCD longest-first order
 ]
 
 
@@ -214,3 +215,44 @@ def test_bwd_block_head_dim_64():
     _check_grad("dk", dkv[0], rdk)
     _check_grad("dv", dkv[1], rdv)
     _check_grad("dq_acc", acc - 0.5, rdq)
+
+
+def test_bwd_block_strided_views_without_copies():
+    """The call site of the generated backward (utils/attn_bwd_dsl.py:83-115): q / out / dout are views of larger
+    buffers (here: a head slice) while block_dq comes from torch.empty, contiguous.  dq and out have stride
+    triples of their own in the C ABI, so the operator makes no contiguous copies of anything."""
+    import mercury_artifact_amd as M
+
+    B, Sq, Sc, H, D = 1, 192, 256, 2, 128
+    g = torch.Generator().manual_seed(14)
+    big = {n: torch.randn(B, Sq, 2 * H, D, generator=g).bfloat16() for n in ("q", "dout")}
+    kv = torch.randn(2, B, Sc, H, D, generator=g).bfloat16()
+    q, dout = big["q"][:, :, H:], big["dout"][:, :, H:]
+    scale = D ** -0.5
+    o, lse = O.block_attention(q.float(), kv[0].float(), kv[1].float(), scale)
+    rdq, rdk, rdv = O.block_backward(dout.float(), q.float(), kv[0].float(), kv[1].float(), o.bfloat16().float(), lse, scale)
+    qd, dd = big["q"].cuda()[:, :, H:], big["dout"].cuda()[:, :, H:]
+    obig = torch.zeros(B, Sq, 3 * H, D, dtype=torch.bfloat16, device="cuda")
+    od = obig[:, :, H:2 * H]
+    od.copy_(o.bfloat16())
+    kvd = kv.cuda()
+    dq = torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device="cuda")          # contiguous, like block_dq
+    dkv = torch.empty_like(kvd)
+    copies = []
+    real = torch.Tensor.contiguous
+
+    def spy(self, *a, **kw):
+        if not self.is_contiguous():
+            copies.append(tuple(self.shape))
+        return real(self, *a, **kw)
+
+    torch.Tensor.contiguous = spy
+    try:
+        M.attn_bwd_block(dd, qd, kvd[0], kvd[1], od, lse.cuda(), dq, dkv[0], dkv[1], scale)
+    finally:
+        torch.Tensor.contiguous = real
+    torch.cuda.synchronize()
+    assert copies == []
+    _check_grad("dq", dq, rdq)
+    _check_grad("dk", dkv[0], rdk)
+    _check_grad("dv", dkv[1], rdv)

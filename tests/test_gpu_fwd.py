@@ -58,6 +58,7 @@ SHAPES = [
     (1, 384, 1100, 2, 1, False),    # 18 tiles, ragged: the four-stage LDS ring wraps several times
     (1, 384, 1100, 2, 1, True),
     (1, 257, 63, 1, 1, False),      # one ragged tile, a second workgroup with a single row
+    (2, 600, 600, 8, 4, True),      # causal with B*Hq a multiple of 8: the per-XCD longest-first order
 ]
 
 

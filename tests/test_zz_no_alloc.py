@@ -28,6 +28,7 @@ def _call(entry, q, k, v, out, lse, dout, scale, causal, with_acc):
     args = [N.ptr(dout), N.ptr(q), N.ptr(k), N.ptr(v), N.ptr(out), N.ptr(lse), N.ptr(dq), N.ptr(dkv[0]), N.ptr(dkv[1]),
             N.ptr(dq_acc), B, Sq, Sc, Hq, Hkv, D, q.stride(0), q.stride(1), q.stride(2),
             k.stride(0), k.stride(1), k.stride(2), dkv[0].stride(0), dkv[0].stride(1), dkv[0].stride(2),
+            dq.stride(0), dq.stride(1), dq.stride(2), out.stride(0), out.stride(1), out.stride(2),
             scale, 1 if causal else 0, 0]
     stream = N.stream_of(q)
     if entry == "workspace":
@@ -71,6 +72,7 @@ def test_no_alloc_entry_rejects_what_does_not_fit():
     # 2^20 + 1 rows: refused before anything is launched (the pointers are never used)
     code = lib.mhip_attn_bwd_block_noalloc(P, P, P, P, P, P, P, P, P, None, 1, (1 << 20) + 1, 64, 1, 1, 128,
                                            ((1 << 20) + 1) * 128, 128, 128, 64 * 128, 128, 128, 64 * 128, 128, 128,
+                                           ((1 << 20) + 1) * 128, 128, 128, ((1 << 20) + 1) * 128, 128, 128,
                                            0.1, 0, 0, None)
     assert code == ETOOLARGE
     assert b"scratch" in lib.mhip_error_string(code)
