@@ -103,6 +103,33 @@ def mfma_ceiling(torch, N, dev, cus):
     return out
 
 
+def operand_dependence(torch, M, dev, shape, scale):
+    """The headline block kernel (one chunk, 4096 x 4096) on operands that toggle few bits: all zeros, and small
+    integers.  Same kernel, same instruction stream, same number of MFMAs; only the switching activity of the
+    data differs, and with it the clock the power management allows."""
+    B, Sq, H, D = shape
+    out = {}
+    flops = 4.0 * B * H * Sq * Sq * D
+    for name, make in (("zeros", lambda *s: torch.zeros(*s, device=dev)),
+                       ("small_integers", lambda *s: torch.randint(-2, 3, s, device=dev).float())):
+        q = make(B, Sq, H, D).bfloat16()
+        kv = make(2, B, Sq, H, D).bfloat16()
+        o = torch.empty_like(q)
+        lse = torch.empty(B, H, Sq, dtype=torch.float32, device=dev)
+        for _ in range(5):
+            M.attn_fwd_block(q, kv[0], kv[1], scale, out=o, lse=lse)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(20):
+            M.attn_fwd_block(q, kv[0], kv[1], scale, out=o, lse=lse)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / 20
+        out[name] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
+                     "pct_of_bf16_mfma_peak": round(flops / ms / 1e9 / PEAK_BF16_TFLOPS * 100, 2)}
+    return out
+
+
 def smi_snapshot():
     """Socket power and clocks as `amd-smi metric --power --clock` prints them, read while the GPU is busy (the
     caller has work queued).  Best effort: None when the tool is missing or refuses."""
@@ -435,6 +462,7 @@ def main() -> int:
     }
     result["sustained"] = sustained
     result["mfma_ceiling"] = mfma_ceiling(torch, M._native, dev, props.multi_processor_count)
+    result["forward_kernel_on_low_toggle_operands"] = operand_dependence(torch, M, dev, (B, Sq, H, D), scale)
     if variants is not None:
         result["other_kernels"] = variants
     if args.cpu_heads > 0:

@@ -76,7 +76,7 @@ __global__ __launch_bounds__(256) void bwd_prepare(const uint16_t* __restrict__ 
 #pragma unroll
   for (int m = 8; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 16);
   if (row < rows && c == 0) {      // (B, Hq, Sq) contiguous
-    delta[row] = acc;
+    delta[row] = -acc;       // stored negated: the main kernels start dP^T = Y Z^T from it (C operand of the first MFMA)
     const float l = lse[row];
     lse2[row] = (l == -INFINITY) ? INFINITY : l * kLog2e;
   }
@@ -269,9 +269,12 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
   auto read_rm = [&](const int (&rm)[8], int mb, int i) -> bf16x8 {
     return *(lds_bf16x8)(uintptr_t)(uint32_t)(rm[i >> 1] + mb * 8192 + ((i & 1) ? kOffY : 0));
   };
+  // T2 starts from -delta of the half's streamed rows (dQ pass: of this lane's stationary row), so that what
+  // the vector unit receives is dP - delta already
+  f32x16 nd;
   auto t_mfma = [&](int i, const bf16x8& a, f32x16& n1, f32x16& n2) {
     const int kk = i >> 1;
-    if (i & 1) n2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, yf[kk], kk == 0 ? zero : n2, 0, 0, 0);
+    if (i & 1) n2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, yf[kk], kk == 0 ? nd : n2, 0, 0, 0);
     else n1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, xf[kk], kk == 0 ? zero : n1, 0, 0, 0);
   };
   // LDS byte addresses of the operand reads for the tile in `stage`
@@ -295,7 +298,7 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
   bf16x8 ring[kDepth];
   f32x16 ta1, ta2, tb1, tb2;      // T1 / T2 of the two halves in flight: (t, first half), (t, second half)
   int rm_c[8], tr_c[4][2], rm_n[8], tr_n[4][2];
-  f32x4 lv[5], dv[5];             // lse2 / delta of 4 streamed rows per entry (dK / dV pass), read one group ahead
+  f32x4 lv[5];                    // lse2 of 4 streamed rows per entry (dK / dV pass), read one group ahead
 
   // Hidden elements (rows past the end of the streamed tensor, the causal mask) get a score of -inf,
   // hence P = dS = 0.  Only the last tile of a head and the tiles the diagonal crosses need it.
@@ -313,19 +316,26 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     }
   };
   // lse2 / delta of rows 8 g + 4 hf .. + 3 of half mb of the tile in `stage`
-  auto read_ld = [&](int stage, int mb, int g, f32x4& l, f32x4& d) {
+  auto read_ld = [&](int stage, int mb, int g, f32x4& l) {
     const int addr = (int)lds_base + stage * kStageBytes + kOffLse + (mb * 32 + g * 8 + hf * 4) * 4;
     l = *(lds_f32x4)(uintptr_t)(uint32_t)addr;
-    d = *(lds_f32x4)(uintptr_t)(uint32_t)(addr + (kOffDelta - kOffLse));
+  };
+  // -delta of rows 8 g + 4 hf .. + 3 (g = 0..3) of half mb of the tile in `stage`, in the order of the
+  // accumulator registers of T2 (dK / dV pass), one group per call
+  auto read_nd = [&](int stage, int mb, int g) {
+    const int addr = (int)lds_base + stage * kStageBytes + kOffDelta + (mb * 32 + g * 8 + hf * 4) * 4;
+    const f32x4 d = *(lds_f32x4)(uintptr_t)(uint32_t)addr;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) nd[4 * g + e] = d[e];
   };
   // P / dS of the half in (c1, c2): 16 accumulator registers, spread over the 16 slots in which the next
   // half's T1 / T2 are issued AND the first slots of the accumulate phase that follows (a wavefront issues
   // one vector instruction every ~5 cycles, so 16 slots of 32 cycles do not hold all of it).  Register e
   // enters at slot first_slot(e); its work is a three-stage pipeline so that no instruction waits for the
   // one issued just before it:
-  //   first_slot      argument of the exponential, dP - delta
+  //   first_slot      argument of the exponential
   //   first_slot + 1  exponential
-  //   first_slot + 2  dS = P (dP - delta)
+  //   first_slot + 2  dS = P (dP - delta)     (c2 arrives as dP - delta)
   // Registers 0-7 (k-step 0 of the accumulate phase) are packed before that phase starts, registers 8-15
   // before its second half does.
   auto first_slot = [](int e) -> int {
@@ -339,11 +349,9 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
       const int f = first_slot(e);
       if (s == f) {
         const float l = DQ ? lse2_lane : lv[e >> 2][e & 3];
-        const float d = DQ ? delta_lane : dv[e >> 2][e & 3];
         earg[e] = __builtin_fmaf(c1[e], p.scale_log2, -l);
-        c2[e] = c2[e] - d;
-        // lse2 / delta of the next four rows, one group ahead
-        if (!DQ && (e & 3) == 0 && e < 12) read_ld(stage, mb, (e >> 2) + 1, lv[(e >> 2) + 1], dv[(e >> 2) + 1]);
+        // lse2 of the next four rows, one group ahead
+        if (!DQ && (e & 3) == 0 && e < 12) read_ld(stage, mb, (e >> 2) + 1, lv[(e >> 2) + 1]);
       }
       if (s == f + 1) c1[e] = fast_exp2(earg[e]);
       if (s == f + 2) c2[e] = c1[e] * c2[e];
@@ -412,6 +420,13 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     static_assert(kCopiesPerTile == (DQ ? 8 : 9), "the vmcnt immediates are one and two tiles of copies");
     __builtin_amdgcn_s_barrier();
     tile_addrs(0, rm_c, tr_c);
+    if (DQ) {
+#pragma unroll
+      for (int j = 0; j < 16; ++j) nd[j] = delta_lane;
+    } else {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) read_nd(0, 0, g);
+    }
     // T1 / T2 of the first half of tile 0, nothing to interleave with
 #pragma unroll
     for (int i = 0; i < kDepth; ++i) ring[i] = read_rm(rm_c, 0, i);
@@ -422,7 +437,11 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     }
 #pragma unroll
     for (int i = 0; i < kDepth; ++i) ring[i] = read_rm(rm_c, 1, i);      // slots 0 .. 3 of tile 0
-    if (!DQ) read_ld(0, 0, 0, lv[0], dv[0]);
+    if (!DQ) {
+      read_ld(0, 0, 0, lv[0]);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) read_nd(0, 1, g);            // for T2 of the second half, first thing in the loop
+    }
   }
   for (int t = 0; t < ntiles; ++t) {
     const int c0 = tile_row0(t);
@@ -447,7 +466,8 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     for (int i = 0; i < kAcc; ++i) {                     // P1
       if (i < kVecTail) vector_slot(16 + i, ta1, ta2, stage, 0);
       acc_mfma(i, ring[(kP1 + i) % kDepth]);
-      if (!DQ && i == kAcc - 2) read_ld(stage, 1, 0, lv[0], dv[0]);
+      if (!DQ && i == kAcc - 2) read_ld(stage, 1, 0, lv[0]);
+      if (!DQ && i >= 2 && i < 6) read_nd((t + 1) & 3, 0, i - 2);      // T2 of (t+1, first half) starts in P2
       ring[(kP1 + i) % kDepth] = read_slot(kP1 + i + kDepth);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -464,7 +484,8 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     for (int i = 0; i < kAcc; ++i) {                     // P3
       if (i < kVecTail) vector_slot(16 + i, tb1, tb2, stage, 1);
       acc_mfma(i, ring[(kP3 + i) % kDepth]);
-      if (!DQ && i == kAcc - 2) read_ld((t + 1) & 3, 0, 0, lv[0], dv[0]);
+      if (!DQ && i == kAcc - 2) read_ld((t + 1) & 3, 0, 0, lv[0]);
+      if (!DQ && i >= 2 && i < 6) read_nd((t + 1) & 3, 1, i - 2);      // T2 of (t+1, second half): P0 of the next tile
       ring[(kP3 + i) % kDepth] = read_slot(kP3 + i + kDepth);
       __builtin_amdgcn_sched_barrier(0);
     }

@@ -223,8 +223,8 @@ def attn_bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_scale, c
     if dk_w is not dk:
         dk.copy_(dk_w)
         dv.copy_(dv_w)
-    # the workspace starts with delta = rowsum(dout * out), (B, Hq, Sq) fp32
-    return ws[: B * Hq * Sq * 4].view(torch.float32).view(B, Hq, Sq)
+    # the workspace starts with -delta = -rowsum(dout * out), (B, Hq, Sq) fp32
+    return ws[: B * Hq * Sq * 4].view(torch.float32).view(B, Hq, Sq).neg()
 
 
 @torch.library.custom_op("mercury_amd::_flash_attn_backward", mutates_args=("dq", "dk", "dv"),
@@ -254,4 +254,4 @@ def _flash_attn_backward(
     Returns ``softmax_d`` (rowsum(dout * out), (B,Hq,Sq) fp32) like flash-attn does."""
     _check_block_inputs(q, k, v, dropout_p, window_size_left, window_size_right, softcap, alibi_slopes)
     return attn_bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_scale, bool(causal),
-                          bool(deterministic)).clone()
+                          bool(deterministic))
