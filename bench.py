@@ -225,7 +225,8 @@ def main() -> int:
     ap.add_argument("--sustain", type=float, default=1.5,
                     help="seconds of back-to-back steps for the `sustained` figure (0 = skip)")
     ap.add_argument("--no-variants", action="store_true",
-                    help="skip the short timings of the causal, backward and fp8 block kernels")
+                    help="skip everything after the headline step: the short timings of the causal, backward and "
+                         "fp8 block kernels, the MFMA ceiling probe and the low-toggle operand runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one rank's step on ONE GPU (the ring is emulated by local buffer rotation); "
@@ -461,9 +462,9 @@ def main() -> int:
                            "bytes_per_launch": merge_bytes},
     }
     result["sustained"] = sustained
-    result["mfma_ceiling"] = mfma_ceiling(torch, M._native, dev, props.multi_processor_count)
-    result["forward_kernel_on_low_toggle_operands"] = operand_dependence(torch, M, dev, (B, Sq, H, D), scale)
     if variants is not None:
+        result["mfma_ceiling"] = mfma_ceiling(torch, M._native, dev, props.multi_processor_count)
+        result["forward_kernel_on_low_toggle_operands"] = operand_dependence(torch, M, dev, (B, Sq, H, D), scale)
         result["other_kernels"] = variants
     if args.cpu_heads > 0:
         result["cpu_baseline"] = cpu_baseline(args.cpu_heads, B, Sq, D, W)
