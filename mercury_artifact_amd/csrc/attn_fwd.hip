@@ -23,7 +23,8 @@
 //   softmax      : the reference score of a row is fixed by the first tile's row maximum and moves only
 //                  when a later tile would overflow: the row SUMS are watched (one compare per tile),
 //                  not the maxima, so the common path has no maximum, no cross-lane exchange and no
-//                  rescale of O; the matrix phase carries no vector work of its own.
+//                  rescale of O; two of a tile's sixteen pairs of exponentials ride behind the last
+//                  MFMAs of the matrix phase (the vector phase was the longer of the two).
 #include "mhip_common.hpp"
 
 namespace mhip {
