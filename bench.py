@@ -359,6 +359,21 @@ def main() -> int:
     real_merges = merge_events
     merge_ms = sum(e0.elapsed_time(e1) for e0, e1 in real_merges) / max(len(real_merges), 1)
     merge_gbs = merge_bytes / (merge_ms * 1e-3) / 1e9
+    # what an event pair reads around a kernel that does next to nothing (one element), launched the same way
+    # between two other kernels: the part of every bracketed duration above that is not the kernel's own
+    # (reported, not subtracted; it matters for the 30 us merge, not for the forward launch)
+    one = torch.zeros(1, device=dev)
+    tiny = []
+    for _ in range(20):
+        dst_probe = o.float()                    # some preceding work on the stream
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        one.add_(1.0)
+        e1.record()
+        tiny.append((e0, e1))
+        del dst_probe
+    torch.cuda.synchronize()
+    tiny_ms = sorted(e0.elapsed_time(e1) for e0, e1 in tiny)[len(tiny) // 2]
 
     # the drop-in boundary itself: a step function spelled the way the generator spells it (bare names resolved in
     # the exec namespace, update_out_and_lse per chunk, the two epilogue stores), run unchanged in
@@ -459,7 +474,7 @@ def main() -> int:
         "roofline_merge": {"bound": "hbm", "kernel": "lse_merge_kernel", "achieved": round(merge_gbs, 1),
                            "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(merge_gbs / PEAK_HBM_GBS, 4),
                            "traffic": TRAFFIC_MERGE_BYTES, "avg_launch_ms": round(merge_ms, 5), "launches": len(real_merges),
-                           "bytes_per_launch": merge_bytes},
+                           "bytes_per_launch": merge_bytes, "event_pair_around_one_element_kernel_ms": round(tiny_ms, 5)},
     }
     result["sustained"] = sustained
     if variants is not None:
