@@ -173,6 +173,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
 #pragma unroll
     for (int j = 0; j < 16; ++j) o_acc[i][j] = 0.f;
   float m_ref = -INFINITY, l_run = 0.f;      // l_run sums 2^7 P (this lane's half of the keys)
+  i32x8 pf[2] = {};          // P^T operands; pf[ks2]: dwords 0-3 = keys of block 2 ks2, dwords 4-7 = block 2 ks2 + 1
   const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   // Tile t lives in stage t % 4 of the K and the V ring.  An iteration starts by waiting for this
@@ -251,7 +252,6 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
     }
     const float msc = (m_ref == -INFINITY) ? 0.f : m_ref * p.scale_log2 - kPShift;   // exponent of 2^7 P
     float rs = 0.f;
-    i32x8 pf[2];               // pf[ks2]: dwords 0-3 = keys of block 2 ks2, dwords 4-7 = block 2 ks2 + 1
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) {
 #pragma unroll
@@ -262,7 +262,9 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
       }
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
-        int packed = 0;
+        // the first conversion writes the low half and the second the high half of the operand register, so
+        // what it held before (the P of the previous tile) needs no clearing
+        int packed = pf[mb >> 1][(mb & 1) * 4 + w];
         packed = __builtin_amdgcn_cvt_pk_fp8_f32(s[mb][4 * w], s[mb][4 * w + 1], packed, false);
         packed = __builtin_amdgcn_cvt_pk_fp8_f32(s[mb][4 * w + 2], s[mb][4 * w + 3], packed, true);
         pf[mb >> 1][(mb & 1) * 4 + w] = packed;
