@@ -29,7 +29,7 @@ extern "C" {
 #define MHIP_OK              0
 #define MHIP_EINVAL         -1   /* bad size / NULL pointer / bad scale                 */
 #define MHIP_EDTYPE         -2   /* dtype code not supported by this entry point       */
-#define MHIP_EHEADDIM       -3   /* head dimension not supported (128 only)            */
+#define MHIP_EHEADDIM       -3   /* head dimension not supported (see the entry point)  */
 #define MHIP_EALIGN         -4   /* pointer or stride not 16-byte aligned              */
 #define MHIP_ELAUNCH        -5   /* hipLaunchKernel / hipGetLastError reported failure */
 #define MHIP_EUNSUPPORTED   -6   /* feature not implemented (dropout, alibi, window..) */
@@ -55,6 +55,10 @@ const char* mhip_error_string(int code);
  * out has q's element type for MHIP_BF16 and is bf16 for MHIP_E4M3.  Rows that see no key
  * get out = 0 and lse = -inf.  For MHIP_E4M3 the three descales are the per-tensor fp32
  * scales s (x ~ s * x_q); ignored for MHIP_BF16.
+ * Head dimension: MHIP_BF16 any multiple of 8 up to 128 (the kernel computes on 128 columns; for D < 128 the
+ * missing ones are zeros that exist only on chip -- no padded copy, no extra memory traffic -- and the K / V
+ * span Sc * stride of one (batch, head) must stay below 2^30 bytes, MHIP_EUNSUPPORTED beyond); MHIP_E4M3 128.
+ * MHIP_EHEADDIM otherwise.
  */
 int mhip_attn_fwd_block(const void* q, const void* k, const void* v, void* out, float* lse,
                         int B, int Sq, int Sc, int Hq, int Hkv, int D,
@@ -76,6 +80,8 @@ int mhip_attn_fwd_block(const void* q, const void* k, const void* v, void* out, 
  * mhip_attn_bwd_workspace_bytes(...) bytes of device memory.  dq and out have element strides of their own:
  * the call site allocates block_dq with torch.empty (contiguous, utils/attn_bwd_dsl.py:83) while q, out and
  * dout are views of the step's buffers; q and dout, k and v, dk and dv share a stride triple each.
+ * Head dimension: any multiple of 8 up to 128, as for the bf16 forward (for D < 128 the q / dout span of one
+ * batch and the k / v span of one (batch, head) must stay below 2^30 bytes).
  */
 int64_t mhip_attn_bwd_workspace_bytes(int B, int Sq, int Sc, int Hq, int Hkv, int D);
 int mhip_attn_bwd_block(const void* dout, const void* q, const void* k, const void* v,

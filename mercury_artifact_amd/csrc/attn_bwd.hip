@@ -38,12 +38,15 @@ constexpr int kStages = 4;
 constexpr int kSmemBytes = kStages * kStageBytes;      // 133120
 constexpr int kOStride = kD + 8;
 constexpr int kNoTile = 0x7fff0000;   // scalar offset that puts every lane of a copy out of range
+constexpr int kNoColumn = 0x7fff0000; // vector offset with the same effect for one lane (the sum of the two is
+                                      // below 2^32: no wrap)
 
 struct BwdParams {
   const uint16_t* q; const uint16_t* k; const uint16_t* v; const uint16_t* dout;
   const float* lse2; const float* delta;   // both (B, Hq, Sq) fp32, written by bwd_prepare
   uint16_t* dq; uint16_t* dk; uint16_t* dv; float* dq_acc;
   int B, Sq, Sc, Hq, Hkv, group;
+  int D;            // head dimension of the tensors, a multiple of 8 up to kD; columns D .. kD-1 are zeros on chip
   int64_t q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, dk_sb, dk_ss, dk_sh, dq_sb, dq_ss, dq_sh, o_sb, o_ss, o_sh;
   float scale, scale_log2;
   int n_tiles;      // stationary tiles per (batch, head)
@@ -52,17 +55,17 @@ struct BwdParams {
   int heads_per_xcd;   // (batch, stationary head) pairs per XCD when they divide evenly, else 0
 };
 
-// delta = rowsum(dout * out): one row of 128 values per 16 lanes (8 values each); lse2 as described above
+// delta = rowsum(dout * out): one row of D <= 128 values per 16 lanes (8 values each); lse2 as described above
 __global__ __launch_bounds__(256) void bwd_prepare(const uint16_t* __restrict__ dout, const uint16_t* __restrict__ out,
                                                    const float* __restrict__ lse, float* __restrict__ delta,
-                                                   float* __restrict__ lse2, int B, int Sq, int Hq,
+                                                   float* __restrict__ lse2, int B, int Sq, int Hq, int D,
                                                    int64_t sb, int64_t ss, int64_t sh,
                                                    int64_t o_sb, int64_t o_ss, int64_t o_sh) {
   const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   const int64_t rows = (int64_t)B * Hq * Sq;
   const int c = threadIdx.x & 15;
   float acc = 0.f;
-  if (row < rows) {
+  if (row < rows && c * 8 < D) {
     const int s = (int)(row % Sq);
     const int64_t bh = row / Sq;
     const int h = (int)(bh % Hq);
@@ -153,11 +156,11 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     const int hk = hs / p.group;
     xbase = p.k + b * p.k_sb + hk * p.k_sh; ybase = p.v + b * p.k_sb + hk * p.k_sh;
     s_ss = p.k_ss; s_sh = 0;
-    s_bytes = (uint32_t)(((int64_t)(p.Sc - 1) * p.k_ss + kD) * 2);
+    s_bytes = (uint32_t)(((int64_t)(p.Sc - 1) * p.k_ss + p.D) * 2);
   } else {
     xbase = p.q + b * p.q_sb; ybase = p.dout + b * p.q_sb;
     s_ss = p.q_ss; s_sh = p.q_sh;
-    s_bytes = (uint32_t)(((int64_t)(p.Sq - 1) * p.q_ss + (int64_t)(p.Hq - 1) * p.q_sh + kD) * 2);
+    s_bytes = (uint32_t)(((int64_t)(p.Sq - 1) * p.q_ss + (int64_t)(p.Hq - 1) * p.q_sh + p.D) * 2);
   }
   const u32x4 xrs = rsrc_words(xbase, s_bytes);
   const u32x4 yrs = rsrc_words(ybase, s_bytes);
@@ -176,7 +179,10 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
     const int row = 16 * wave + 4 * u + (lane >> 4);
-    cvoff[u] = (int)(row * s_ss * 2) + (((lane & 15) ^ lds_row_swizzle(row)) << 4);
+    const int chunk = (lane & 15) ^ lds_row_swizzle(row);
+    // chunks past the head dimension: an offset that is out of the descriptor's range for every tile, so they
+    // arrive as zeros and a tile in LDS always has 128 columns
+    cvoff[u] = chunk * 8 < p.D ? (int)(row * s_ss * 2) + (chunk << 4) : kNoColumn;
   }
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
   auto copy_tile = [&](int t, int stage) {
@@ -404,8 +410,13 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     }
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
-      xf[ks] = *reinterpret_cast<const bf16x8*>(xp + ks * 16);
-      yf[ks] = *reinterpret_cast<const bf16x8*>(yp + ks * 16);
+      if (ks * 16 + hf * 8 < p.D) {
+        xf[ks] = *reinterpret_cast<const bf16x8*>(xp + ks * 16);
+        yf[ks] = *reinterpret_cast<const bf16x8*>(yp + ks * 16);
+      } else {                                       // columns past the head dimension
+        xf[ks] = bf16x8{};
+        yf[ks] = bf16x8{};
+      }
     }
     // Pin the loads here (the copies are invisible to the compiler's wait counting), the MFMA operands into
     // accumulation registers: the arithmetic registers are needed for the tiles of T1 / T2 that the vector
@@ -517,7 +528,7 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     for (int it = 0; it < 8; ++it) {
       const int r = (lane >> 4) + 4 * it;
       const int row = r0 + wave * 32 + r;
-      if (row < n_st) {
+      if (row < n_st && chunk * 8 < p.D) {
         const u32x4 w = *reinterpret_cast<const u32x4*>(os + r * (kOStride * 2) + chunk * 16);
         *reinterpret_cast<u32x4*>(op + (int64_t)row * d_ss) = w;
       }
@@ -527,16 +538,18 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     write_out(acc1, p.scale, p.dq, p.dq_sb, p.dq_ss, p.dq_sh, hs);
     if (p.dq_acc != nullptr && my_r < n_st) {
       // fp32 accumulator (B, Sq, Hq, D) contiguous; every element belongs to exactly one lane
-      float* ap = p.dq_acc + (((int64_t)b * p.Sq + my_r) * p.Hq + hs) * kD;
+      float* ap = p.dq_acc + (((int64_t)b * p.Sq + my_r) * p.Hq + hs) * p.D;
 #pragma unroll
       for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          f32x4* a4 = reinterpret_cast<f32x4*>(ap + db * 32 + g * 8 + hf * 4);
-          f32x4 v = *a4;
+          if (db * 32 + g * 8 + hf * 4 < p.D) {
+            f32x4* a4 = reinterpret_cast<f32x4*>(ap + db * 32 + g * 8 + hf * 4);
+            f32x4 v = *a4;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] += acc1[db][4 * g + e] * p.scale;
-          *a4 = v;
+            for (int e = 0; e < 4; ++e) v[e] += acc1[db][4 * g + e] * p.scale;
+            *a4 = v;
+          }
         }
     }
   } else {
@@ -598,7 +611,7 @@ int bwd_block(const void* dout, const void* q, const void* k, const void* v,
   if (B < 0 || Sq < 0 || Sc < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return MHIP_EINVAL;
   if (!(softmax_scale > 0.f) || !(softmax_scale < INFINITY)) return MHIP_EINVAL;
   if (mask != MHIP_MASK_NONE && mask != MHIP_MASK_CAUSAL) return MHIP_EINVAL;
-  if (D != kD) return MHIP_EHEADDIM;
+  if (D < 8 || D > kD || (D & 7) != 0) return MHIP_EHEADDIM;     // below 128 the missing columns are zeros on chip
   if (B == 0) return MHIP_OK;
   if (Sq > 0 && (!dout || !q || !out || !lse || !dq || (!workspace && !own_scratch))) return MHIP_EINVAL;
   if (Sc > 0 && (!k || !v || !dk || !dv)) return MHIP_EINVAL;
@@ -613,6 +626,8 @@ int bwd_block(const void* dout, const void* q, const void* k, const void* v,
   const int64_t q_span = ((int64_t)Sq * q_ss + (int64_t)Hq * q_sh) * 2;
   const int64_t k_span = (int64_t)Sc * k_ss * 2;
   if (q_span >= (int64_t(1) << 31) || k_span >= (int64_t(1) << 31)) return MHIP_EUNSUPPORTED;
+  // below 128 the lanes of the missing columns carry the offset kNoColumn, which has to be out of range
+  if (D < kD && (q_span >= (int64_t(1) << 30) || k_span >= (int64_t(1) << 30))) return MHIP_EUNSUPPORTED;
   if (own_scratch && Sq > 0) {
     if ((int64_t)B * Hq * Sq > kScratchRows) return MHIP_ETOOLARGE;
     const int rc = scratch_address(&workspace);
@@ -628,6 +643,7 @@ int bwd_block(const void* dout, const void* q, const void* k, const void* v,
   p.dq = static_cast<uint16_t*>(dq); p.dk = static_cast<uint16_t*>(dk); p.dv = static_cast<uint16_t*>(dv);
   p.dq_acc = dq_acc;
   p.B = B; p.Sq = Sq; p.Sc = Sc; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv;
+  p.D = D;
   p.q_sb = q_sb; p.q_ss = q_ss; p.q_sh = q_sh;
   p.k_sb = k_sb; p.k_ss = k_ss; p.k_sh = k_sh;
   p.dk_sb = dk_sb; p.dk_ss = dk_ss; p.dk_sh = dk_sh;
@@ -640,7 +656,7 @@ int bwd_block(const void* dout, const void* q, const void* k, const void* v,
     const int64_t rows = (int64_t)B * Hq * Sq;
     hipLaunchKernelGGL(bwd_prepare, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
                        static_cast<const uint16_t*>(dout), static_cast<const uint16_t*>(out), lse,
-                       delta_buf, lse2_buf, B, Sq, Hq, q_sb, q_ss, q_sh, o_sb, o_ss, o_sh);
+                       delta_buf, lse2_buf, B, Sq, Hq, D, q_sb, q_ss, q_sh, o_sb, o_ss, o_sh);
     // dQ: one workgroup per 128 query rows
     p.n_tiles = (Sq + kRowsPerWg - 1) / kRowsPerWg;
     p.total = B * Hq * p.n_tiles;

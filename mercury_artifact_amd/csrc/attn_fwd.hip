@@ -38,6 +38,8 @@ constexpr int kTileBytes = kBN * kD * 2;   // 16384: one K or V tile in LDS, 64 
 constexpr int kStages = 4;                 // K(t+1) .. K(t+4) and V(t) .. V(t+3) live while tile t is processed
 constexpr int kVBase = kStages * kTileBytes;
 constexpr int kOStride = kD + 8;   // epilogue staging of O, bf16 elements per row
+constexpr int kNoColumn = 0x7fff0000;  // vector offset that is out of every descriptor's range (spans stay below 2^31,
+                                       // and so does the scalar tile offset added to it: no 32-bit wrap)
 #ifndef MHIP_FWD_FRAG_DEPTH
 #define MHIP_FWD_FRAG_DEPTH 4
 #endif
@@ -47,6 +49,7 @@ struct FwdParams {
   const uint16_t* q; const uint16_t* k; const uint16_t* v;
   uint16_t* out; float* lse;
   int B, Sq, Sc, Hq, Hkv, group;
+  int D;             // head dimension of the tensors, a multiple of 8 up to kD; columns D .. kD-1 are zeros on chip
   int64_t q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, v_sb, v_ss, v_sh, o_sb, o_ss, o_sh;
   float scale, scale_log2;
   int nq_tiles;      // ceil(Sq / rows per workgroup)
@@ -111,17 +114,20 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
   // of a transposing read.  Wavefront w copies rows 8w .. 8w+7 of every tile with two instructions of
   // 1 KB; lane l of instruction u lands at row 8w + 4u + l/16, position l%16 (the hardware places the
   // lanes back to back) and therefore fetches chunk (l%16) ^ swz(row).  Rows past the end of the chunk
-  // are out of the descriptor's range and arrive as zeros.
+  // are out of the descriptor's range and arrive as zeros, and so do the chunks past the head dimension
+  // when it is below 128: their lanes carry an offset that is out of range for every tile, so a tile in
+  // LDS always has 128 columns, the upper ones zero, at no cost in memory traffic.
   auto swz = [](int row) { return lds_row_swizzle(row); };
-  const u32x4 krs = rsrc_words(p.k + b * p.k_sb + hk * p.k_sh, (uint32_t)(((int64_t)(p.Sc - 1) * p.k_ss + kD) * 2));
-  const u32x4 vrs = rsrc_words(p.v + b * p.v_sb + hk * p.v_sh, (uint32_t)(((int64_t)(p.Sc - 1) * p.v_ss + kD) * 2));
+  const u32x4 krs = rsrc_words(p.k + b * p.k_sb + hk * p.k_sh, (uint32_t)(((int64_t)(p.Sc - 1) * p.k_ss + p.D) * 2));
+  const u32x4 vrs = rsrc_words(p.v + b * p.v_sb + hk * p.v_sh, (uint32_t)(((int64_t)(p.Sc - 1) * p.v_ss + p.D) * 2));
   int kvoff[2], vvoff[2];
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const int row = 8 * wave + 4 * u + (lane >> 4);
     const int chunk = (lane & 15) ^ swz(row);
-    kvoff[u] = (int)(row * p.k_ss * 2) + chunk * 16;
-    vvoff[u] = (int)(row * p.v_ss * 2) + chunk * 16;
+    const bool real = chunk * 8 < p.D;
+    kvoff[u] = real ? (int)(row * p.k_ss * 2) + chunk * 16 : kNoColumn;
+    vvoff[u] = real ? (int)(row * p.v_ss * 2) + chunk * 16 : kNoColumn;
   }
   const int k_tile_bytes = (int)(kBN * p.k_ss * 2);
   const int v_tile_bytes = (int)(kBN * p.v_ss * 2);
@@ -342,7 +348,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     const int row = my_q < p.Sq ? my_q : p.Sq - 1;
     const uint16_t* qp = p.q + b * p.q_sb + (int64_t)row * p.q_ss + hq * p.q_sh + hf * 8;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qp + ks * 16);
+    for (int ks = 0; ks < 8; ++ks) {
+      if (ks * 16 + hf * 8 < p.D) qf[ks] = *reinterpret_cast<const bf16x8*>(qp + ks * 16);
+      else qf[ks] = bf16x8{};                       // columns past the head dimension
+    }
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) asm volatile("" : "+v"(qf[ks]));
   }
@@ -409,7 +418,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     for (int it = 0; it < 8; ++it) {
       const int r = (lane >> 4) + 4 * it;
       const int row = q0 + wave * 32 + r;
-      if (row < p.Sq) {
+      if (row < p.Sq && chunk * 8 < p.D) {
         const u32x4 w = *reinterpret_cast<const u32x4*>(os + r * (kOStride * 2) + chunk * 16);
         *reinterpret_cast<u32x4*>(op + (int64_t)row * p.o_ss) = w;
       }
@@ -420,7 +429,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
 }  // namespace
 
 int attn_fwd_bf16(const void* q, const void* k, const void* v, void* out, float* lse,
-                  int B, int Sq, int Sc, int Hq, int Hkv,
+                  int B, int Sq, int Sc, int Hq, int Hkv, int D,
                   const int64_t* st, float scale, int mask, hipStream_t stream) {
   FwdParams p;
   p.q = static_cast<const uint16_t*>(q);
@@ -429,6 +438,7 @@ int attn_fwd_bf16(const void* q, const void* k, const void* v, void* out, float*
   p.out = static_cast<uint16_t*>(out);
   p.lse = lse;
   p.B = B; p.Sq = Sq; p.Sc = Sc; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv;
+  p.D = D;
   p.q_sb = st[0]; p.q_ss = st[1]; p.q_sh = st[2];
   p.k_sb = st[3]; p.k_ss = st[4]; p.k_sh = st[5];
   p.v_sb = st[6]; p.v_ss = st[7]; p.v_sh = st[8];

@@ -65,38 +65,19 @@ def _host_scalar(t) -> float:
     return value
 
 
-_KERNEL_D = 128
-
-
-def _paddable(D: int) -> bool:
-    return 0 < D < _KERNEL_D and D % 8 == 0
-
-
-def _pad_d(t: torch.Tensor) -> torch.Tensor:
-    """``t`` with its last dimension zero-padded to the kernels' head dimension (a new contiguous tensor)."""
-    return torch.nn.functional.pad(t, (0, _KERNEL_D - t.shape[-1]))
-
-
 def attn_fwd_block(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float,
                    causal: bool = False, q_descale: Optional[torch.Tensor] = None,
                    k_descale: Optional[torch.Tensor] = None, v_descale: Optional[torch.Tensor] = None,
                    out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
                    ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """(Q shard, one KV chunk) -> (out (B,Sq,Hq,D), lse (B,Hq,Sq) fp32) through mhip_attn_fwd_block."""
+    """(Q shard, one KV chunk) -> (out (B,Sq,Hq,D), lse (B,Hq,Sq) fp32) through mhip_attn_fwd_block.
+    bfloat16: any head dimension that is a multiple of 8 up to 128 (the kernels work on 128 columns and fill the
+    missing ones with zeros on chip, which changes neither the scores nor the columns that exist);
+    float8_e4m3fn: 128."""
     _check_block_inputs(q, k, v, 0, -1, -1, 0.0, None)
     N.require_cuda(out, lse, q_descale, k_descale, v_descale)
     B, Sq, Hq, D = q.shape
     _, Sc, Hkv, _ = k.shape
-    if q.dtype == torch.bfloat16 and _paddable(D):
-        # head dimensions below 128: the kernels are built for D = 128, and zero columns change neither the
-        # scores nor the columns that matter, so the block runs on zero-padded copies (correct, not fast)
-        po, lse = attn_fwd_block(_pad_d(q), _pad_d(k), _pad_d(v), softmax_scale, causal, lse=lse)
-        if out is None:
-            return po[..., :D].contiguous(), lse
-        if out.shape != (B, Sq, Hq, D) or out.dtype != torch.bfloat16:
-            raise RuntimeError("out must be (B, Sq, Hq, D) bfloat16 with a contiguous last dimension")
-        out.copy_(po[..., :D])
-        return out, lse
     if q.dtype == torch.bfloat16:
         dt, out_dtype = N.MHIP_BF16, torch.bfloat16
     elif q.dtype == torch.float8_e4m3fn:
@@ -172,17 +153,6 @@ def attn_bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_scale, c
     _, Sc, Hkv, _ = k.shape
     if q.dtype != torch.bfloat16:
         raise RuntimeError("the backward kernel takes bfloat16 only")
-    if _paddable(D) and all(t.dtype == torch.bfloat16 for t in (dout, out, dq, dk, dv)):
-        # as in the forward: zero-padded copies; the gradients of the padded columns are exactly zero
-        pdq, pdk, pdv = (torch.empty(t.shape[:-1] + (_KERNEL_D,), dtype=t.dtype, device=t.device) for t in (q, k, v))
-        acc = None if dq_acc is None else torch.zeros(dq_acc.shape[:-1] + (_KERNEL_D,), dtype=torch.float32,
-                                                      device=q.device)
-        delta = attn_bwd_block(_pad_d(dout), _pad_d(q), _pad_d(k), _pad_d(v), _pad_d(out), softmax_lse, pdq, pdk, pdv,
-                               softmax_scale, causal, deterministic, dq_acc=acc)
-        dq.copy_(pdq[..., :D]); dk.copy_(pdk[..., :D]); dv.copy_(pdv[..., :D])
-        if dq_acc is not None:
-            dq_acc.add_(acc[..., :D])
-        return delta
     for name, t, like in (("dout", dout, q), ("out", out, q), ("dq", dq, q), ("dk", dk, k), ("dv", dv, k)):
         if t.shape != like.shape or t.dtype != torch.bfloat16:
             raise RuntimeError(f"{name} must be bfloat16 with shape {tuple(like.shape)}")

@@ -24,7 +24,12 @@ def _fwd(lib, q=P, k=P, v=P, out=P, lse=P, B=1, Sq=64, Sc=64, Hq=2, Hkv=2, D=128
 
 
 def test_forward_rejects(lib):
-    assert _fwd(lib, D=64) == EHEADDIM
+    for bad in (0, 4, 100, 136, 256):
+        assert _fwd(lib, D=bad) == EHEADDIM
+    assert _fwd(lib, D=64, dtype=1) == EHEADDIM                 # e4m3: 128 only
+    big64 = 1 << 19                                             # D = 64: spans of one (batch, head) stay below 1 GiB
+    assert _fwd(lib, D=64, Sc=1024, strides=[64 * 128, 128, 64, 1024 * big64, big64, 64, 1024 * big64, big64, 64,
+                                             64 * 128, 128, 64]) == EUNSUPPORTED
     assert _fwd(lib, Hq=3, Hkv=2) == EINVAL
     assert _fwd(lib, Sq=-1) == EINVAL
     assert _fwd(lib, scale=0.0) == EINVAL
@@ -56,7 +61,8 @@ def test_backward_rejects(lib):
         return lib.mhip_attn_bwd_block(P, P, P, P, P, P, dq, P, P, dq_acc, B, Sq, Sc, Hq, Hkv, D, *strides,
                                        scale, mask, 0, ws, None)
 
-    assert bwd(D=96) == EHEADDIM
+    for bad in (0, 4, 100, 136, 256):
+        assert bwd(D=bad) == EHEADDIM
     assert bwd(Hq=5, Hkv=2) == EINVAL
     assert bwd(scale=-1.0) == EINVAL
     assert bwd(mask=3) == EINVAL

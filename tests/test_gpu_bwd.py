@@ -202,7 +202,7 @@ def test_bwd_ring_full_size(fused):
 
 
 def test_bwd_block_head_dim_64():
-    """Head dimension 64 through the backward (zero-padded operands, gradients of the padding dropped)."""
+    """Head dimension 64 through the backward (the missing columns are zeros on chip only)."""
     import mercury_artifact_amd as M
 
     q, kv, dout, o16, lse, scale, (rdq, rdk, rdv) = _case(2, 160, 200, 4, 2, True, seed=12, D=64)
@@ -215,6 +215,39 @@ def test_bwd_block_head_dim_64():
     _check_grad("dk", dkv[0], rdk)
     _check_grad("dv", dkv[1], rdv)
     _check_grad("dq_acc", acc - 0.5, rdq)
+
+
+@pytest.mark.parametrize("D", [64, 24])
+def test_bwd_block_small_head_dim_reads_and_writes_only_its_columns(D):
+    """Every tensor of the block backward as a column slice of a 128-wide one: NaN next to the inputs, a sentinel
+    next to the outputs.  Nothing outside the D columns may be fetched or stored."""
+    import mercury_artifact_amd as M
+
+    B, Sq, Sc, Hq, Hkv = 1, 160, 200, 4, 2
+    q, kv, dout, o16, lse, scale, (rdq, rdk, rdv) = _case(B, Sq, Sc, Hq, Hkv, False, seed=15, D=D)
+    off = 128 - D
+
+    def wide(t, fill):
+        w = torch.full(t.shape[:-1] + (128,), fill, dtype=torch.bfloat16, device="cuda")
+        w[..., off:].copy_(t.cuda())
+        return w, w[..., off:]
+
+    nan = float("nan")
+    (_, qv), (_, dv_), (_, ov) = wide(q, nan), wide(dout, nan), wide(o16, nan)
+    kvw = torch.full((2, B, Sc, Hkv, 128), nan, dtype=torch.bfloat16, device="cuda")
+    kvw[..., off:].copy_(kv.cuda())
+    kvv = kvw[..., off:]
+    dqw = torch.full((B, Sq, Hq, 128), 7.0, dtype=torch.bfloat16, device="cuda")
+    dkvw = torch.full((2, B, Sc, Hkv, 128), 7.0, dtype=torch.bfloat16, device="cuda")
+    acc = torch.full((B, Sq, Hq, D), 0.5, dtype=torch.float32, device="cuda")
+    M.attn_bwd_block(dv_, qv, kvv[0], kvv[1], ov, lse.cuda(), dqw[..., off:], dkvw[0][..., off:], dkvw[1][..., off:],
+                     scale, dq_acc=acc)
+    torch.cuda.synchronize()
+    _check_grad("dq", dqw[..., off:], rdq)
+    _check_grad("dk", dkvw[0][..., off:], rdk)
+    _check_grad("dv", dkvw[1][..., off:], rdv)
+    _check_grad("dq_acc", acc - 0.5, rdq)
+    assert (dqw[..., :off] == 7.0).all() and (dkvw[..., :off] == 7.0).all()
 
 
 def test_bwd_block_strided_views_without_copies():

@@ -158,6 +158,33 @@ def test_fwd_block_strided_views_and_guard_bands():
     assert (lbuf[:pad] == 7.0).all() and (lbuf[-pad:] == 7.0).all()
 
 
+@pytest.mark.parametrize("D", [64, 40])
+def test_fwd_block_small_head_dim_reads_and_writes_only_its_columns(D):
+    """q, k, v and out as COLUMN slices of 128-wide tensors whose other columns hold NaN (inputs) or a sentinel
+    (output): a kernel that fetched or stored its full 128 on-chip columns would pick up the NaN or clobber the
+    sentinel.  The slices keep the 128-element head stride, so nothing is copied on the way in."""
+    import mercury_artifact_amd as M
+
+    B, Sq, Sc, Hq, Hkv = 1, 200, 330, 4, 2
+    q, kv = _mk(B, Sq, Sc, Hq, Hkv, D=D, seed=33)
+    scale = D ** -0.5
+    ro, rl = O.block_attention(q.float(), kv[0].float(), kv[1].float(), scale, causal=True)
+    qw = torch.full((B, Sq, Hq, 128), float("nan"), dtype=torch.bfloat16, device="cuda")
+    kvw = torch.full((2, B, Sc, Hkv, 128), float("nan"), dtype=torch.bfloat16, device="cuda")
+    ow = torch.full((B, Sq, Hq, 128), 7.0, dtype=torch.bfloat16, device="cuda")
+    for off in (0, 128 - D):                                    # the slice at the left and at the right edge
+        qw.fill_(float("nan")); kvw.fill_(float("nan")); ow.fill_(7.0)
+        qv, kvv, ov = qw[..., off:off + D], kvw[..., off:off + D], ow[..., off:off + D]
+        qv.copy_(q.cuda()); kvv.copy_(kv.cuda())
+        out, lse = M.attn_fwd_block(qv, kvv[0], kvv[1], scale, causal=True, out=ov)
+        torch.cuda.synchronize()
+        assert out is ov
+        _check(ov, lse, ro, rl, f"D{D} off{off}")
+        rest = torch.ones(128, dtype=torch.bool)
+        rest[off:off + D] = False
+        assert (ow[..., rest.cuda()] == 7.0).all()
+
+
 def test_fwd_rejects_what_it_does_not_implement():
     import mercury_artifact_amd as M
 
@@ -207,9 +234,10 @@ def test_fwd_chunks_merge_to_single_pass_full_size():
     _check(o[:, :, heads], lse[:, heads], ro, rl, "config1")
 
 
-@pytest.mark.parametrize("D,causal", [(64, False), (64, True), (32, False), (96, True)])
+@pytest.mark.parametrize("D,causal", [(64, False), (64, True), (32, False), (96, True), (8, False), (120, True)])
 def test_fwd_block_smaller_head_dims(D, causal):
-    """Head dimensions below 128 (multiples of 8) run through the same kernel on zero-padded operands."""
+    """Head dimensions below 128 (multiples of 8) run through the same kernel: the columns that do not exist are
+    zeros on chip only (no padded copies)."""
     import mercury_artifact_amd as M
 
     B, Sq, Sc, Hq, Hkv = 2, 200, 330, 4, 2
