@@ -1,6 +1,6 @@
 """Seeded random small shapes through the three block kernels and the one-pass fold against the CPU oracle: ragged row and key
-counts, batch 1-3, 1-4 query heads per KV head, with and without the causal mask.  Tolerances as in the
-per-kernel test files."""
+counts, batch 1-3, 1-4 query heads per KV head, with and without the causal mask, and (bf16) a head dimension drawn
+from the multiples of 8 up to 128, half of the cases 128.  Tolerances as in the per-kernel test files."""
 import random
 
 import pytest
@@ -21,15 +21,24 @@ def _shapes(seed, n, max_s):
     return out
 
 
+def _head_dim(*key):
+    seed = 0
+    for k in key:
+        seed = seed * 1000003 + int(k)
+    rng = random.Random(seed)
+    return 128 if rng.random() < 0.5 else 8 * rng.randint(1, 15)
+
+
 @pytest.mark.parametrize("B,Sq,Sc,Hq,Hkv,causal", _shapes(101, 16, 420))
 def test_random_forward(B, Sq, Sc, Hq, Hkv, causal):
     import mercury_artifact_amd as M
 
-    print(f"fwd B{B} Sq{Sq} Sc{Sc} Hq{Hq} Hkv{Hkv} causal={causal}", flush=True)
+    D = _head_dim(B, Sq, Sc, Hq)
+    print(f"fwd B{B} Sq{Sq} Sc{Sc} Hq{Hq} Hkv{Hkv} D{D} causal={causal}", flush=True)
     g = torch.Generator().manual_seed(B * 1000003 + Sq * 1009 + Sc)
-    q = torch.randn(B, Sq, Hq, 128, generator=g).bfloat16()
-    kv = torch.randn(2, B, Sc, Hkv, 128, generator=g).bfloat16()
-    scale = 128 ** -0.5
+    q = torch.randn(B, Sq, Hq, D, generator=g).bfloat16()
+    kv = torch.randn(2, B, Sc, Hkv, D, generator=g).bfloat16()
+    scale = D ** -0.5
     ro, rl = O.block_attention(q.float(), kv[0].float(), kv[1].float(), scale, causal=causal)
     out, lse = M.attn_fwd_block(q.cuda(), kv[0].cuda(), kv[1].cuda(), scale, causal=causal)
     out, lse = out.float().cpu(), lse.cpu()
@@ -46,12 +55,13 @@ def test_random_forward(B, Sq, Sc, Hq, Hkv, causal):
 def test_random_backward(B, Sq, Sc, Hq, Hkv, causal):
     import mercury_artifact_amd as M
 
-    print(f"bwd B{B} Sq{Sq} Sc{Sc} Hq{Hq} Hkv{Hkv} causal={causal}", flush=True)
+    D = _head_dim(B, Sq, Sc, Hq, 7)
+    print(f"bwd B{B} Sq{Sq} Sc{Sc} Hq{Hq} Hkv{Hkv} D{D} causal={causal}", flush=True)
     g = torch.Generator().manual_seed(B * 1000003 + Sq * 1009 + Sc + 7)
-    q = torch.randn(B, Sq, Hq, 128, generator=g).bfloat16()
-    kv = torch.randn(2, B, Sc, Hkv, 128, generator=g).bfloat16()
-    dout = torch.randn(B, Sq, Hq, 128, generator=g).bfloat16()
-    scale = 128 ** -0.5
+    q = torch.randn(B, Sq, Hq, D, generator=g).bfloat16()
+    kv = torch.randn(2, B, Sc, Hkv, D, generator=g).bfloat16()
+    dout = torch.randn(B, Sq, Hq, D, generator=g).bfloat16()
+    scale = D ** -0.5
     o, lse = O.block_attention(q.float(), kv[0].float(), kv[1].float(), scale, causal=causal)
     o16 = o.bfloat16()
     refs = O.block_backward(dout.float(), q.float(), kv[0].float(), kv[1].float(), o16.float(), lse, scale,
