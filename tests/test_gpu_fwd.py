@@ -253,7 +253,7 @@ def test_fwd_block_smaller_head_dims(D, causal):
 
 
 def test_config0_through_the_gpu_path():
-    """BASELINE configuration 0 (the CPU plumbing case: B1 H4 D64, Q 1024 x 4 KV chunks of 256, N(0,1) from
+    """The smallest benchmark configuration (the CPU plumbing case: B1 H4 D64, Q 1024 x 4 KV chunks of 256, N(0,1) from
     torch.manual_seed(0), scale 1/8) through libmercury_hip.so: the inputs are rounded to bf16 (the block
     operator takes no fp32, like the flash-attn operator it replaces) and every rank's ring step -- one fold,
     the literal chain, and unchanged generated-style text in the lazy namespace -- is compared with single-pass
