@@ -55,8 +55,8 @@ const char* mhip_error_string(int code);
  * out has q's element type for MHIP_BF16 and is bf16 for MHIP_E4M3.  Rows that see no key
  * get out = 0 and lse = -inf.  For MHIP_E4M3 the three descales are the per-tensor fp32
  * scales s (x ~ s * x_q); ignored for MHIP_BF16.
- * Head dimension: MHIP_BF16 any multiple of 8 up to 128 (the kernel computes on 128 columns; for D < 128 the
- * missing ones are zeros that exist only on chip -- no padded copy, no extra memory traffic -- and the K / V
+ * Head dimension: MHIP_BF16 any multiple of 8 up to 128 (the kernel computes on 128 columns, on 64 for D <= 64;
+ * the missing ones are zeros that exist only on chip -- no padded copy, no extra memory traffic -- and the K / V
  * span Sc * stride of one (batch, head) must stay below 2^30 bytes, MHIP_EUNSUPPORTED beyond); MHIP_E4M3 128.
  * MHIP_EHEADDIM otherwise.
  */

@@ -58,8 +58,14 @@ struct FwdParams {
   int heads_per_xcd; // (batch, head) pairs per XCD when they divide evenly, else 0
 };
 
-template <bool CAUSAL>
+// KK = k-steps of 16 head-dim values in S^T: 8 computes on all 128 on-chip columns; 4 is the instantiation for head
+// dimensions up to 64, which leaves out the MFMAs that would only see the zero columns (half of both products).
+template <bool CAUSAL, int KK = 8>
 __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdParams p) {
+  static_assert(KK == 8 || KK == 4, "128 or 64 on-chip head-dim columns");
+  constexpr int DB = KK / 2;        // blocks of 32 head-dim values in O^T
+  constexpr int kSlotsS = 2 * KK;   // matrix-phase slots of S^T (two 32-key blocks per k-step)
+  constexpr int kSlotsO = 4 * DB;   // and of O^T (four k-steps of 16 keys per block)
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kStages * kTileBytes];
 
   // Workgroup i runs on XCD i % 8.  Give every XCD a contiguous range of the (batch, head, q-tile)
@@ -106,7 +112,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
 
   // ---- Q fragment: B operand of S^T = K Q^T, lane (ln, hf) holds Q[row][16 ks + 8 hf .. +7] -----
   const int my_q = q0 + wave * 32 + ln;
-  bf16x8 qf[8];   // loaded in the prologue, after the first tile copies are under way
+  bf16x8 qf[KK];  // loaded in the prologue, after the first tile copies are under way
 
   // ---- global -> LDS copies of the K and V tiles ---------------------------------------------------
   // A tile is 64 rows of 256 bytes.  Chunk c (16 bytes) of row r lives at chunk position c ^ swz(r):
@@ -144,19 +150,19 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
 
   // K operand of S^T (A, 32 keys x 16 head-dim values): lane (ln, hf) reads chunk 2 kk + hf of row
   // 32 mb + ln.
-  int k_rd[8];                                        // + mb * 8192
+  int k_rd[KK];                                       // + mb * 8192
 #pragma unroll
-  for (int kk = 0; kk < 8; ++kk) k_rd[kk] = ln * 256 + (((2 * kk + hf) ^ swz(ln)) << 4);
+  for (int kk = 0; kk < KK; ++kk) k_rd[kk] = ln * 256 + (((2 * kk + hf) ^ swz(ln)) << 4);
   // V^T operand of O^T (A, 32 head-dim values x 16 keys) for head-dim block db and k-step (mb, j2): the
   // lane's 8 keys are rows R + {0..3} and R + 8 + {0..3}, R = 32 mb + 16 j2 + 4 hf -- the keys its P
   // registers hold.  One ds_read_b64_tr_b16 per group of 4 rows: within 16 lanes, lane s supplies the
   // address of row R + s/4, head-dim values 4 (s%4) .. +3 of the 16-column strip, and receives column s.
-  int v_rd[4][2];                                     // [db][second four rows]  + mb * 8192 + j2 * 4096
+  int v_rd[DB][2];                                    // [db][second four rows]  + mb * 8192 + j2 * 4096
   {
     const int s16 = lane & 15, strip = (lane >> 4) & 1;
     const int cl = 2 * strip + ((s16 & 3) >> 1);
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+    for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         const int row = 8 * h + 4 * hf + (s16 >> 2);
@@ -176,9 +182,9 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
   const int causal_shift = p.Sc - p.Sq;
 
   // ---- accumulators -----------------------------------------------------------------------------
-  f32x16 o_acc[4];
+  f32x16 o_acc[DB];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < DB; ++i)
 #pragma unroll
     for (int j = 0; j < 16; ++j) o_acc[i][j] = 0.f;
   // m_ref: the raw (unscaled) score the exponentials of this lane's Q row are taken relative to.  It is
@@ -196,7 +202,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
   auto qk = [&](int stage) {
     const unsigned char* ks = smem + stage * kTileBytes;
 #pragma unroll
-    for (int kk = 0; kk < 8; ++kk) {
+    for (int kk = 0; kk < KK; ++kk) {
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb) {
         const bf16x8 kf = read_k(ks, mb, kk);
@@ -210,7 +216,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
 #pragma unroll
     for (int kstep = 0; kstep < 4; ++kstep) {
 #pragma unroll
-      for (int db = 0; db < 4; ++db) {
+      for (int db = 0; db < DB; ++db) {
         const bf16x8 vf = read_v(vs, db, kstep);
         o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, __builtin_bit_cast(bf16x8, pw[kstep]), o_acc[db], 0, 0, 0);
       }
@@ -269,7 +275,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     if (!first) {
       const float alpha = move ? fast_exp2(-grown) : 1.f;
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+      for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int j = 0; j < 16; ++j) o_acc[db][j] *= alpha;
       l_run *= alpha;
@@ -281,12 +287,16 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
 #define MHIP_FWD_EARLY_PAIRS 2
 #endif
   constexpr int kEarlyPairs = MHIP_FWD_EARLY_PAIRS;
-  // slot of the matrix phase after which early pair idx runs: k-step idx / 4 of the tile before is read by
-  // slots 16 + 4 (idx / 4) .. + 3, and the pairs are spread two slots apart behind that
+  // slot of the matrix phase after which early pair idx runs: k-step idx / 4 of the tile before is read by the
+  // O^T slots kSlotsS + DB (idx / 4) .. + DB - 1, and the pairs are spread two slots apart behind that
 #ifndef MHIP_FWD_EARLY_STEP
 #define MHIP_FWD_EARLY_STEP 2
 #endif
-  auto early_slot = [](int idx) { return idx < 4 ? 20 + MHIP_FWD_EARLY_STEP * idx : 28 + (idx - 4); };
+  auto early_slot = [](int idx) {
+    return idx < 4 ? kSlotsS + DB + MHIP_FWD_EARLY_STEP * idx : kSlotsS + 3 * DB + (idx - 4);
+  };
+  static_assert(kEarlyPairs <= 4 && kSlotsS + DB + MHIP_FWD_EARLY_STEP * (kEarlyPairs - 1) < kSlotsS + kSlotsO,
+                "the early pairs have to fit behind the O^T slots of k-step 0");
   auto sm_tile = [&]() {
 #pragma unroll
     for (int idx = kEarlyPairs; idx < 16; ++idx) sm_pair(idx);
@@ -298,11 +308,11 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
   };
 
   // Matrix phase of tile t: S^T(t+1) from K stage `ks_stage` and O^T += V^T(t) P^T(t) from V stage
-  // `vs_stage`, 32 MFMAs fed by 32 LDS reads.  The reads run kFragDepth operands ahead of the MFMAs
-  // through a ring of registers, so the LDS latency is covered by the MFMAs in between.
+  // `vs_stage`, kSlotsS + kSlotsO MFMAs (32 on 128 columns) fed by as many LDS reads.  The reads run kFragDepth
+  // operands ahead of the MFMAs through a ring of registers, so the LDS latency is covered by the MFMAs in between.
   auto read_frag = [&](int i, const unsigned char* ks, const unsigned char* vs) -> bf16x8 {
-    if (i < 16) return read_k(ks, i & 1, i >> 1);
-    return read_v(vs, (i - 16) & 3, (i - 16) >> 2);
+    if (i < kSlotsS) return read_k(ks, i & 1, i >> 1);
+    return read_v(vs, (i - kSlotsS) % DB, (i - kSlotsS) / DB);
   };
   // The first kFragDepth operands (all of K) are read before the barrier that opens the phase, by
   // first_frags, so the matrix pipe starts without waiting for LDS.
@@ -316,17 +326,17 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     const unsigned char* ks = smem + ks_stage * kTileBytes;
     const unsigned char* vs = smem + kVBase + vs_stage * kTileBytes;
 #pragma unroll
-    for (int i = 0; i < 32; ++i) {
-      if (i < 16) {
+    for (int i = 0; i < kSlotsS + kSlotsO; ++i) {
+      if (i < kSlotsS) {
         const int mb = i & 1, kk = i >> 1;
         s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag[i % kFragDepth], qf[kk], kk == 0 ? zero : s[mb], 0, 0, 0);
       } else {
-        const int db = (i - 16) & 3, kstep = (i - 16) >> 2;
+        const int db = (i - kSlotsS) % DB, kstep = (i - kSlotsS) / DB;
         o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag[i % kFragDepth], __builtin_bit_cast(bf16x8, pw[kstep]), o_acc[db], 0, 0, 0);
       }
-      if (i + kFragDepth < 32) frag[i % kFragDepth] = read_frag(i + kFragDepth, ks, vs);
-      // S^T(t_next) is complete after slot 15; its softmax starts here, in the shadow of the O^T MFMAs
-      if (i == 16) sm_mask(t_next);
+      if (i + kFragDepth < kSlotsS + kSlotsO) frag[i % kFragDepth] = read_frag(i + kFragDepth, ks, vs);
+      // S^T(t_next) is complete after its last slot; its softmax starts here, in the shadow of the O^T MFMAs
+      if (i == kSlotsS) sm_mask(t_next);
 #pragma unroll
       for (int idx = 0; idx < kEarlyPairs; ++idx)
         if (early_slot(idx) == i) sm_pair(idx);
@@ -348,12 +358,12 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     const int row = my_q < p.Sq ? my_q : p.Sq - 1;
     const uint16_t* qp = p.q + b * p.q_sb + (int64_t)row * p.q_ss + hq * p.q_sh + hf * 8;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
+    for (int ks = 0; ks < KK; ++ks) {
       if (ks * 16 + hf * 8 < p.D) qf[ks] = *reinterpret_cast<const bf16x8*>(qp + ks * 16);
       else qf[ks] = bf16x8{};                       // columns past the head dimension
     }
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) asm volatile("" : "+v"(qf[ks]));
+    for (int ks = 0; ks < KK; ++ks) asm volatile("" : "+v"(qf[ks]));
   }
   if (ntiles > 0) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -402,7 +412,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
   __syncthreads();   // every wave is done with the K/V tiles: reuse LDS to transpose O
   unsigned char* os = smem + wave * (32 * kOStride * 2);
 #pragma unroll
-  for (int db = 0; db < 4; ++db)
+  for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       u32x2 w;
@@ -450,10 +460,14 @@ int attn_fwd_bf16(const void* q, const void* k, const void* v, void* out, float*
   p.per_xcd = (p.total + 7) / 8;
   p.heads_per_xcd = (B * Hq) % 8 == 0 ? (B * Hq) / 8 : 0;
   const dim3 grid(p.per_xcd * 8), block(kWaves * 64);
-  if (mask == MHIP_MASK_CAUSAL)
-    hipLaunchKernelGGL(attn_fwd_bf16_d128<true>, grid, block, 0, stream, p);
-  else
-    hipLaunchKernelGGL(attn_fwd_bf16_d128<false>, grid, block, 0, stream, p);
+  const bool causal = mask == MHIP_MASK_CAUSAL;
+  if (D <= 64) {        // half the on-chip columns, half the MFMAs
+    if (causal) hipLaunchKernelGGL((attn_fwd_bf16_d128<true, 4>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((attn_fwd_bf16_d128<false, 4>), grid, block, 0, stream, p);
+  } else {
+    if (causal) hipLaunchKernelGGL((attn_fwd_bf16_d128<true, 8>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((attn_fwd_bf16_d128<false, 8>), grid, block, 0, stream, p);
+  }
   return launch_status();
 }
 
