@@ -57,8 +57,8 @@ const char* mhip_error_string(int code);
  * scales s (x ~ s * x_q); ignored for MHIP_BF16.
  * Head dimension: MHIP_BF16 any multiple of 8 up to 128 (the kernel computes on 128 columns, on 64 for D <= 64;
  * the missing ones are zeros that exist only on chip -- no padded copy, no extra memory traffic -- and the K / V
- * span Sc * stride of one (batch, head) must stay below 2^30 bytes, MHIP_EUNSUPPORTED beyond); MHIP_E4M3 128.
- * MHIP_EHEADDIM otherwise.
+ * span Sc * stride of one (batch, head) must stay below 2^30 bytes, MHIP_EUNSUPPORTED beyond); MHIP_E4M3 any
+ * multiple of 16 up to 128, in the same way.  MHIP_EHEADDIM otherwise.
  */
 int mhip_attn_fwd_block(const void* q, const void* k, const void* v, void* out, float* lse,
                         int B, int Sq, int Sc, int Hq, int Hkv, int D,

@@ -7,7 +7,7 @@ int attn_fwd_bf16(const void* q, const void* k, const void* v, void* out, float*
                   int B, int Sq, int Sc, int Hq, int Hkv, int D,
                   const int64_t* strides, float scale, int mask, hipStream_t stream);
 int attn_fwd_fp8(const void* q, const void* k, const void* v, void* out, float* lse,
-                 int B, int Sq, int Sc, int Hq, int Hkv, const int64_t* strides, float scale, int mask,
+                 int B, int Sq, int Sc, int Hq, int Hkv, int D, const int64_t* strides, float scale, int mask,
                  float q_descale, float k_descale, float v_descale, hipStream_t stream);
 }  // namespace mhip
 
@@ -20,7 +20,7 @@ extern "C" const char* mhip_error_string(int code) {
     case MHIP_OK: return "ok";
     case MHIP_EINVAL: return "invalid argument (size, NULL pointer or softmax scale)";
     case MHIP_EDTYPE: return "element type not supported by this entry point";
-    case MHIP_EHEADDIM: return "head dimension not supported (bf16: a multiple of 8 up to 128; e4m3: 128)";
+    case MHIP_EHEADDIM: return "head dimension not supported (bf16: a multiple of 8 up to 128; e4m3: a multiple of 16 up to 128)";
     case MHIP_EALIGN: return "pointer or stride not aligned to 16 bytes";
     case MHIP_ELAUNCH: return "kernel launch failed";
     case MHIP_EUNSUPPORTED: return "feature not implemented";
@@ -47,8 +47,8 @@ extern "C" int mhip_attn_fwd_block(const void* q, const void* k, const void* v, 
   if (!(softmax_scale > 0.f) || !(softmax_scale < INFINITY)) return MHIP_EINVAL;
   if (mask != MHIP_MASK_NONE && mask != MHIP_MASK_CAUSAL) return MHIP_EINVAL;
   if (dtype != MHIP_BF16 && dtype != MHIP_E4M3) return MHIP_EDTYPE;
-  // bf16: any multiple of 8 up to 128 (the kernel works on 128 columns, the missing ones zero on chip); e4m3: 128
-  if (dtype == MHIP_E4M3 ? D != 128 : (D < 8 || D > 128 || (D & 7) != 0)) return MHIP_EHEADDIM;
+  // any multiple of 8 (bf16) or of 16 (e4m3) up to 128: the kernels work on 128 columns, the missing ones zero on chip
+  if (D <= 0 || D > 128 || (D & (dtype == MHIP_E4M3 ? 15 : 7)) != 0) return MHIP_EHEADDIM;
   if (B == 0 || Sq == 0) return MHIP_OK;
   if (!q || !out || !lse) return MHIP_EINVAL;
   if (Sc > 0 && (!k || !v)) return MHIP_EINVAL;
@@ -69,7 +69,7 @@ extern "C" int mhip_attn_fwd_block(const void* q, const void* k, const void* v, 
   const int64_t strides[12] = {q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, v_sb, v_ss, v_sh, o_sb, o_ss, o_sh};
   if (fp8) {
     if (!(q_descale > 0.f) || !(k_descale > 0.f) || !(v_descale > 0.f)) return MHIP_EINVAL;
-    return attn_fwd_fp8(q, k, v, out, lse, B, Sq, Sc, Hq, Hkv, strides, softmax_scale, mask,
+    return attn_fwd_fp8(q, k, v, out, lse, B, Sq, Sc, Hq, Hkv, D, strides, softmax_scale, mask,
                         q_descale, k_descale, v_descale, st);
   }
   return attn_fwd_bf16(q, k, v, out, lse, B, Sq, Sc, Hq, Hkv, D, strides, softmax_scale, mask, st);

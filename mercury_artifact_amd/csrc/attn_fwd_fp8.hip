@@ -35,11 +35,14 @@ constexpr int kVBase = kStages * kTileBytes;
 constexpr int kOStride = kD + 8;
 constexpr float kPShift = 7.f;        // P is stored as 2^7 P in e4m3
 constexpr float kRescaleSlack = 1.f;
+constexpr int kNoColumn = 0x7fff0000;  // vector offset that is out of every descriptor's range (spans stay below 2^30
+                                       // when it is used, and so does the scalar tile offset added to it)
 
 struct Fp8Params {
   const uint8_t* q; const uint8_t* k; const uint8_t* v;
   uint16_t* out; float* lse;
   int B, Sq, Sc, Hq, Hkv, group;
+  int D;             // head dimension of the tensors, a multiple of 16 up to kD; columns D .. kD-1 are zeros on chip
   int64_t q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, v_sb, v_ss, v_sh, o_sb, o_ss, o_sh;
   float scale_eff;       // softmax_scale * q_descale * k_descale: natural-log scale of the integer-like dot
   float scale_log2;      // scale_eff * log2(e)
@@ -101,15 +104,18 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
   // ---- global -> LDS copies: wavefront w copies rows 16w .. 16w+15 of every K and V tile with two
   // instructions of 1 KB; lane l of instruction u lands at row 16w + 8u + l/8, chunk position l%8, and
   // fetches the chunk that lives there.  Rows past the end of the chunk arrive as zeros. ---------------------
-  const u32x4 krs = rsrc_words(p.k + b * p.k_sb + hk * p.k_sh, (uint32_t)((int64_t)(p.Sc - 1) * p.k_ss + kD));
-  const u32x4 vrs = rsrc_words(p.v + b * p.v_sb + hk * p.v_sh, (uint32_t)((int64_t)(p.Sc - 1) * p.v_ss + kD));
+  // Chunks past the head dimension (D < 128) carry an offset that is out of range for every tile and arrive as
+  // zeros too: a tile in LDS always has 128 columns, at no cost in memory traffic.
+  const u32x4 krs = rsrc_words(p.k + b * p.k_sb + hk * p.k_sh, (uint32_t)((int64_t)(p.Sc - 1) * p.k_ss + p.D));
+  const u32x4 vrs = rsrc_words(p.v + b * p.v_sb + hk * p.v_sh, (uint32_t)((int64_t)(p.Sc - 1) * p.v_ss + p.D));
   int kvoff[2], vvoff[2];
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const int row = 16 * wave + 8 * u + (lane >> 3);
     const int chunk = (lane & 7) ^ swz8(row);
-    kvoff[u] = (int)(row * p.k_ss) + chunk * 16;
-    vvoff[u] = (int)(row * p.v_ss) + chunk * 16;
+    const bool real = chunk * 16 < p.D;
+    kvoff[u] = real ? (int)(row * p.k_ss) + chunk * 16 : kNoColumn;
+    vvoff[u] = real ? (int)(row * p.v_ss) + chunk * 16 : kNoColumn;
   }
   const int k_tile_bytes = (int)(kBN * p.k_ss);
   const int v_tile_bytes = (int)(kBN * p.v_ss);
@@ -190,8 +196,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
     const uint8_t* qp = p.q + b * p.q_sb + (int64_t)row * p.q_ss + hq * p.q_sh + hf * 32;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      const u32x4 lo = *reinterpret_cast<const u32x4*>(qp + ks * 64);
-      const u32x4 hi = *reinterpret_cast<const u32x4*>(qp + ks * 64 + 16);
+      const u32x4 none = {0u, 0u, 0u, 0u};                        // columns past the head dimension
+      const int col = ks * 64 + hf * 32;
+      const u32x4 lo = col < p.D ? *reinterpret_cast<const u32x4*>(qp + ks * 64) : none;
+      const u32x4 hi = col + 16 < p.D ? *reinterpret_cast<const u32x4*>(qp + ks * 64 + 16) : none;
 #pragma unroll
       for (int e = 0; e < 4; ++e) { qf[ks][e] = (int)lo[e]; qf[ks][4 + e] = (int)hi[e]; }
     }
@@ -310,7 +318,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
     for (int it = 0; it < 8; ++it) {
       const int r = (lane >> 4) + 4 * it;
       const int row = q0 + wave * 32 + r;
-      if (row < p.Sq) {
+      if (row < p.Sq && chunk * 8 < p.D) {
         const u32x4 w = *reinterpret_cast<const u32x4*>(os + r * (kOStride * 2) + chunk * 16);
         *reinterpret_cast<u32x4*>(op + (int64_t)row * p.o_ss) = w;
       }
@@ -321,12 +329,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
 }  // namespace
 
 int attn_fwd_fp8(const void* q, const void* k, const void* v, void* out, float* lse,
-                 int B, int Sq, int Sc, int Hq, int Hkv, const int64_t* st, float scale, int mask,
+                 int B, int Sq, int Sc, int Hq, int Hkv, int D, const int64_t* st, float scale, int mask,
                  float q_descale, float k_descale, float v_descale, hipStream_t stream) {
   Fp8Params p;
   p.q = static_cast<const uint8_t*>(q); p.k = static_cast<const uint8_t*>(k); p.v = static_cast<const uint8_t*>(v);
   p.out = static_cast<uint16_t*>(out); p.lse = lse;
   p.B = B; p.Sq = Sq; p.Sc = Sc; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv;
+  p.D = D;
   p.q_sb = st[0]; p.q_ss = st[1]; p.q_sh = st[2];
   p.k_sb = st[3]; p.k_ss = st[4]; p.k_sh = st[5];
   p.v_sb = st[6]; p.v_ss = st[7]; p.v_sh = st[8];

@@ -73,7 +73,7 @@ def attn_fwd_block(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_sc
     """(Q shard, one KV chunk) -> (out (B,Sq,Hq,D), lse (B,Hq,Sq) fp32) through mhip_attn_fwd_block.
     bfloat16: any head dimension that is a multiple of 8 up to 128 (the kernels work on 128 columns and fill the
     missing ones with zeros on chip, which changes neither the scores nor the columns that exist);
-    float8_e4m3fn: 128."""
+    float8_e4m3fn: any multiple of 16 up to 128, in the same way."""
     _check_block_inputs(q, k, v, 0, -1, -1, 0.0, None)
     N.require_cuda(out, lse, q_descale, k_descale, v_descale)
     B, Sq, Hq, D = q.shape

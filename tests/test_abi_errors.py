@@ -26,7 +26,7 @@ def _fwd(lib, q=P, k=P, v=P, out=P, lse=P, B=1, Sq=64, Sc=64, Hq=2, Hkv=2, D=128
 def test_forward_rejects(lib):
     for bad in (0, 4, 100, 136, 256):
         assert _fwd(lib, D=bad) == EHEADDIM
-    assert _fwd(lib, D=64, dtype=1) == EHEADDIM                 # e4m3: 128 only
+    assert _fwd(lib, D=72, dtype=1) == EHEADDIM                 # e4m3: multiples of 16
     big64 = 1 << 19                                             # D = 64: spans of one (batch, head) stay below 1 GiB
     assert _fwd(lib, D=64, Sc=1024, strides=[64 * 128, 128, 64, 1024 * big64, big64, 64, 1024 * big64, big64, 64,
                                              64 * 128, 128, 64]) == EUNSUPPORTED

@@ -70,6 +70,39 @@ def test_fp8_block_matches_oracle(B, Sq, Sc, Hq, Hkv, causal):
     _check(out, lse, ref_a, ref_b, "fp8 block", p_bound, check_b=Sc >= 1000)
 
 
+@pytest.mark.parametrize("D,causal", [(64, False), (48, True), (16, False), (112, True)])
+def test_fp8_block_smaller_head_dims(D, causal):
+    """Head dimensions below 128 (multiples of 16) through the e4m3 kernel: q, k, v and out are COLUMN slices of
+    128-wide tensors whose other columns hold the e4m3 NaN code (inputs) or a sentinel (output), so a kernel that
+    fetched or stored its full 128 on-chip columns would pick up the NaN or clobber the sentinel."""
+    import mercury_artifact_amd as M
+
+    B, Sq, Sc, Hq, Hkv = 1, 200, 330, 4, 2
+    print(f"fp8 small head dim D{D} causal={causal}", flush=True)
+    (q, k, v), (qq, kq, vq), (sq, sk, sv) = _quantised(B, Sq, Sc, Hq, Hkv, seed=40 + D, D=D)
+    scale = D ** -0.5
+    deq = (O.dequantize(qq, sq), O.dequantize(kq, sk), O.dequantize(vq, sv))
+    ref_a = O.block_attention(*deq, scale, causal=causal)
+    ref_b = O.block_attention(q, k, v, scale, causal=causal)
+    off = 128 - D
+    nan8 = torch.full((1,), float("nan")).to(torch.float8_e4m3fn)
+
+    def wide(t):
+        w = nan8.cuda().expand(t.shape[:-1] + (128,)).contiguous()
+        view = w[..., off:]
+        view.copy_(t.cuda())
+        return view
+
+    qv, kv_, vv = wide(qq), wide(kq), wide(vq)
+    ow = torch.full((B, Sq, Hq, 128), 7.0, dtype=torch.bfloat16, device="cuda")
+    out, lse = M.attn_fwd_block(qv, kv_, vv, scale, causal=causal, q_descale=sq.cuda(), k_descale=sk.cuda(),
+                                v_descale=sv.cuda(), out=ow[..., off:])
+    torch.cuda.synchronize()
+    p_bound = O.e4m3_p_rounding_bound(*deq, scale, causal=causal)
+    _check(out, lse, ref_a, ref_b, f"fp8 D{D}", p_bound, check_b=False)
+    assert (ow[..., :off] == 7.0).all()
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", [(4, 300, 3, 128), (1003,), (7,), (2, 4099)])
 def test_fp8_product_quantiser_bits(dtype, shape):
