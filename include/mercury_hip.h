@@ -156,7 +156,7 @@ int mhip_lse_merge(const float* acc_out, const float* acc_lse,
  * block_outs[i] bf16 (B, Sq - s_begin[i], Hq, D) addressed with the element strides bo_sb[i], bo_ss, bo_sh
  * (multiples of 8, 16-byte aligned base, D contiguous), block_lses[i] fp32 (B, Hq, Sq - s_begin[i])
  * contiguous.  final_out bf16 (B,Sq,Hq,D) contiguous, final_lse fp32 (B,Hq,Sq) contiguous.
- * D in {64, 128, 256}.  Rows whose lse is -inf in every block get (0, -inf).
+ * D a multiple of 8 up to 256.  Rows whose lse is -inf in every block get (0, -inf).
  */
 int mhip_lse_merge_many(const void* const* block_outs, const float* const* block_lses,
                         const int64_t* bo_sb, const int* s_begin, int n,

@@ -482,19 +482,21 @@ struct MergeManyParams {
   int s_begin[kMaxBlocks];        // first sequence row the block covers
   int64_t bo_sb[kMaxBlocks];      // batch stride of the block's output, elements
   int n, Sq, Hq;
+  int D;                          // head dimension, a multiple of 8; a row takes LPR >= D / 8 lanes (a power of two)
   int64_t rows;
   int64_t bo_ss, bo_sh;
 };
 
 template <int LPR, int N>          // N = 0: run-time block count, folded in groups of kGroup
 __global__ __launch_bounds__(256) void lse_merge_many_kernel(const MergeManyParams p) {
-  constexpr int D = LPR * 8;
+  const int D = p.D;
   constexpr int kRowsPerPass = 256 / LPR;
   constexpr int G = N > 0 ? N : kGroup;
   const int n = N > 0 ? N : p.n;
   const int64_t row = (int64_t)blockIdx.x * kRowsPerPass + threadIdx.x / LPR;
   if (row >= p.rows) return;
   const int col = (threadIdx.x % LPR) * 8;
+  if (col >= D) return;            // head dimensions that do not fill the row's lanes (no cross-lane work below)
   const uint32_t h = (uint32_t)row % (uint32_t)p.Hq;
   const uint32_t bs = (uint32_t)row / (uint32_t)p.Hq;
   const uint32_t s = bs % (uint32_t)p.Sq;
@@ -658,7 +660,7 @@ extern "C" int mhip_lse_merge_many(const void* const* block_outs, const float* c
                                    int B, int Sq, int Hq, int D,
                                    int64_t bo_ss, int64_t bo_sh, void* stream) {
   if (B < 0 || Sq < 0 || Hq < 0 || D <= 0 || n < 1 || n > kMaxBlocks) return MHIP_EINVAL;
-  if (D != 64 && D != 128 && D != 256) return MHIP_EUNSUPPORTED;
+  if (D > 256 || (D & 7) != 0) return MHIP_EUNSUPPORTED;
   const int64_t rows = (int64_t)B * Sq * Hq;
   if (rows == 0) return MHIP_OK;
   if (rows >= (int64_t(1) << 31)) return MHIP_EUNSUPPORTED;
@@ -678,14 +680,14 @@ extern "C" int mhip_lse_merge_many(const void* const* block_outs, const float* c
     p.lse[i] = block_lses[i];
   }
   p.final_out = static_cast<uint16_t*>(final_out); p.final_lse = final_lse;
-  p.n = n; p.Sq = Sq; p.Hq = Hq; p.rows = rows;
+  p.n = n; p.Sq = Sq; p.Hq = Hq; p.D = D; p.rows = rows;
   p.bo_ss = bo_ss; p.bo_sh = bo_sh;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  switch (D) {
-    case 64: launch_merge_many<8>(p, st); break;
-    case 128: launch_merge_many<16>(p, st); break;
-    default: launch_merge_many<32>(p, st); break;
-  }
+  // lanes per row: the power of two that holds D / 8 (all lanes busy at D = 32, 64, 128, 256)
+  if (D <= 32) launch_merge_many<4>(p, st);
+  else if (D <= 64) launch_merge_many<8>(p, st);
+  else if (D <= 128) launch_merge_many<16>(p, st);
+  else launch_merge_many<32>(p, st);
   return launch_status();
 }
 

@@ -95,7 +95,7 @@ def test_elementwise_rejects(lib):
     assert many(outs=(ctypes.c_void_p * 2)(P, P + 8)) == EALIGN
     assert many(st=(128 * 4 + 4, 128)) == EALIGN
     assert many(sb=(ctypes.c_int64 * 2)(4096, 4100)) == EALIGN
-    assert many(D=40) == EUNSUPPORTED
+    assert many(D=44) == EUNSUPPORTED and many(D=264) == EUNSUPPORTED      # multiples of 8 up to 256
     assert many(B=0) == OK
     assert lib.mhip_tree_merge(P, None, P, 8, 128, 0, None) == EINVAL
     assert lib.mhip_tree_merge(P + 8, P, P, 8, 128, 1, None) == EALIGN

@@ -219,7 +219,7 @@ def test_add_collective_sums_the_group():
 
 
 @pytest.mark.parametrize("n", [1, 2, 3, 8, 16, 17, 32, 45, 64])
-@pytest.mark.parametrize("B,Sq,H,D", [(2, 37, 3, 128), (1, 64, 4, 64), (1, 9, 2, 256)])
+@pytest.mark.parametrize("B,Sq,H,D", [(2, 37, 3, 128), (1, 64, 4, 64), (1, 9, 2, 256), (2, 21, 3, 96), (1, 50, 2, 8)])
 def test_merge_many_matches_the_chain(n, B, Sq, H, D):
     """One fold of all block results against the chain of reference merges in fp64 followed by the
     epilogue.  The output is bf16: atol 1e-3 + rtol 2^-8 (one bf16 rounding of the result); lse 1e-5."""

@@ -109,7 +109,7 @@ def test_random_fp8_forward(B, Sq, Sc, Hq, Hkv, causal):
 
 def _fold_cases(seed, n):
     rng = random.Random(seed)
-    return [(rng.randint(1, 3), rng.randint(1, 300), rng.randint(1, 6), rng.choice([64, 128, 256]), rng.randint(1, 16))
+    return [(rng.randint(1, 3), rng.randint(1, 300), rng.randint(1, 6), rng.choice([64, 128, 256, 128, 96, 40, 8, 200]), rng.randint(1, 16))
             for _ in range(n)]
 
 

@@ -57,6 +57,27 @@ def test_single_ring_reference_test_shape(rank, fused, deferred):
     assert torch.equal(qd, q_before) and torch.equal(dev_kvs[rank], kv_before)   # inputs untouched
 
 
+@pytest.mark.parametrize("D", [96, 40, 64])
+@pytest.mark.parametrize("deferred", [True, False])
+def test_single_ring_other_head_dims(D, deferred):
+    """The ring drivers at head dimensions other than 128: block kernels on zero-filled on-chip columns, the fold
+    (or the chain of merges) on D-wide rows."""
+    import mercury_artifact_amd as M
+
+    B, S, H, W, rank = 2, 1024, 3, 4, 2
+    q, k, v, qs, kvs = _inputs(B, S, H, H, D, W, seed=9)
+    scale = D ** -0.5
+    ro, rl = O.single_pass_attention(qs[rank].float(), k.float(), v.float(), scale)
+    dev_kvs = [c.cuda() for c in kvs]
+    qd = qs[rank].cuda()
+    o = torch.empty_like(qd)
+    lse = torch.empty(B, H, S // W, dtype=torch.float32, device="cuda")
+    M.flash_attn_pack_kv(qd, dev_kvs[rank], o, lse, scale, ring=M.LocalRing((W,), rank, dev_kvs),
+                         deferred_merge=deferred, fused_epilogue=deferred)
+    torch.cuda.synchronize()
+    _compare(o, lse, ro, rl)
+
+
 @pytest.mark.parametrize("divide,deferred", [(2, True), (4, True), (4, False), (8, True), (16, True)])
 def test_single_ring_with_ring_divide(divide, deferred):
     """ring_divide = k (tests/test_ring_attn_codegen.py:102, benchmark/bench_attn.py:178): k * W block calls on
