@@ -42,17 +42,19 @@ struct MergeParams {
   float* dst_out; float* dst_lse;
   uint16_t* final_out; float* final_lse;
   int B, Sq, Hq;
+  int D;             // head dimension (the vector kernels: a multiple of 4; a row takes LPR >= D / 4 lanes)
   int64_t rows;
   int64_t ao_sb, ao_ss, ao_sh, al_sb, al_ss, al_sh, bo_sb, bo_ss, bo_sh, bl_sb, bl_sh;
   int64_t do_sb, do_ss, do_sh, dl_sb, dl_ss, dl_sh;
 };
 
-// One row = LPR lanes x 4 contiguous head-dim values, ROWS rows per thread.  Measured on MI355X at
+// One row = LPR lanes x 4 contiguous head-dim values (lanes past the head dimension idle: LPR is the power of two
+// that holds D / 4), ROWS rows per thread.  Measured on MI355X at
 // 131072 rows x 128: two rows per thread with non-temporal stores is the fastest setting (5.8 TB/s in
 // place, 5.2 TB/s into a separate destination); more rows per thread or non-temporal loads are slower.
 template <int LPR, int ROWS, bool FIRST, bool FINAL>
 __global__ __launch_bounds__(256) void lse_merge_kernel(const MergeParams p) {
-  constexpr int D = LPR * 4;
+  const int D = p.D;
   constexpr int kRowsPerPass = 256 / LPR;
   const int sub = threadIdx.x / LPR;
   const int col = (threadIdx.x % LPR) * 4;
@@ -73,7 +75,7 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const MergeParams p) {
 #pragma unroll
   for (int r = 0; r < ROWS; ++r) {
     const int64_t row = row0 + (int64_t)r * kRowsPerPass;
-    live[r] = row < p.rows;
+    live[r] = row < p.rows && col < D;
     if (r > 0) {
       h += kRowsPerPass;
       while (h >= (uint32_t)p.Hq) {
@@ -204,7 +206,7 @@ __global__ __launch_bounds__(256) void lse_merge_kernel8(const MergeParams p) {
 #pragma unroll
   for (int r = 0; r < ROWS; ++r) {
     const int64_t row = row0 + (int64_t)r * kRowsPerPass;
-    live[r] = row < p.rows;
+    live[r] = row < p.rows && col < D;
     if (r > 0) {
       h += kRowsPerPass;
       while (h >= (uint32_t)p.Hq) {
@@ -621,7 +623,8 @@ extern "C" int mhip_lse_merge(const float* acc_out, const float* acc_lse,
   hipStream_t st = static_cast<hipStream_t>(stream);
   // the vector kernel needs 16-byte aligned fp32 rows and 8-byte aligned bf16 rows
   auto mult4 = [](int64_t x) { return (x & 3) == 0; };
-  bool vec = (D == 32 || D == 64 || D == 128 || D == 256) && p.rows < (int64_t(1) << 31) &&
+  p.D = D;
+  bool vec = (D & 3) == 0 && D <= 256 && p.rows < (int64_t(1) << 31) &&
              mult4(bo_sb) && mult4(bo_ss) && mult4(bo_sh) &&
              (reinterpret_cast<uintptr_t>(block_out) & 7u) == 0;
   if (!first) vec = vec && mult4(ao_sb) && mult4(ao_ss) && mult4(ao_sh) && aligned16(acc_out);
@@ -636,12 +639,11 @@ extern "C" int mhip_lse_merge(const float* acc_out, const float* acc_lse,
   if (vec8) {
     launch_merge8<16>(p, first, fin, st);
   } else if (vec) {
-    switch (D) {
-      case 32: launch_merge<8>(p, first, fin, st); break;
-      case 64: launch_merge<16>(p, first, fin, st); break;
-      case 128: launch_merge<32>(p, first, fin, st); break;
-      default: launch_merge<64>(p, first, fin, st); break;
-    }
+    // lanes per row: the power of two that holds D / 4 (all lanes busy at D = 32, 64, 128, 256)
+    if (D <= 32) launch_merge<8>(p, first, fin, st);
+    else if (D <= 64) launch_merge<16>(p, first, fin, st);
+    else if (D <= 128) launch_merge<32>(p, first, fin, st);
+    else launch_merge<64>(p, first, fin, st);
   } else {
     constexpr int kRowsPerBlock = 256 / kGenericLanes;
     if (p.rows / kRowsPerBlock >= (int64_t(1) << 31)) return MHIP_EUNSUPPORTED;
