@@ -53,12 +53,13 @@ def test_update_out_and_lse_matches_reference_formula(B, Sq, H, D):
         M.update_out_and_lse(None, None, bod, bld, slice_=(slice(None), slice(0, 1)))
 
 
-@pytest.mark.parametrize("D", [40, 130])
+@pytest.mark.parametrize("D", [40, 130, 42])
 def test_merge_in_place_generic_head_dim_beyond_residency(D):
-    """dst == acc on the path taken for head dimensions other than 32/64/128/256 (one row per 32 lanes of one
-    wavefront: the row's lse is read by all its lanes before the one store), at a row count whose grid is far
-    larger than what is resident at once, so that rows merged late would see lse values stored early if any
-    thread read an lse it does not own."""
+    """dst == acc at head dimensions other than 32/64/128/256: multiples of 4 take the vector kernel with idle
+    lanes (40), everything else (130, 42) the generic one (one row per 32 lanes of one wavefront: the row's lse
+    is read by all its lanes before the one store).  The row count makes the grid far larger than what is
+    resident at once, so that rows merged late would see lse values stored early if any thread read an lse it
+    does not own."""
     import mercury_artifact_amd as M
 
     B, Sq, H = 2, 40000, 3
