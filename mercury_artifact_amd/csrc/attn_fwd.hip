@@ -40,10 +40,9 @@ constexpr int kVBase = kStages * kTileBytes;
 constexpr int kOStride = kD + 8;   // epilogue staging of O, bf16 elements per row
 constexpr int kNoColumn = 0x7fff0000;  // vector offset that is out of every descriptor's range (spans stay below 2^31,
                                        // and so does the scalar tile offset added to it: no 32-bit wrap)
-#ifndef MHIP_FWD_FRAG_DEPTH
-#define MHIP_FWD_FRAG_DEPTH 4
-#endif
-constexpr int kFragDepth = MHIP_FWD_FRAG_DEPTH;  // LDS operand reads in flight ahead of the MFMAs
+constexpr int kFragDepth = 4;      // LDS operand reads in flight ahead of the MFMAs (6 and 8 measure the same)
+constexpr int kEarlyPairs = 2;     // exponential pairs of a tile computed inside the matrix phase (4 .. 8: 1-3 % slower)
+constexpr int kEarlyStep = 2;      // matrix-phase slots between them
 
 struct FwdParams {
   const uint16_t* q; const uint16_t* k; const uint16_t* v;
@@ -283,19 +282,12 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_bf16_d128(const FwdPa
     m_ref = move ? mx : m_ref;
     nmsc = -m_ref * p.scale_log2;
   };
-#ifndef MHIP_FWD_EARLY_PAIRS
-#define MHIP_FWD_EARLY_PAIRS 2
-#endif
-  constexpr int kEarlyPairs = MHIP_FWD_EARLY_PAIRS;
   // slot of the matrix phase after which early pair idx runs: k-step idx / 4 of the tile before is read by the
   // O^T slots kSlotsS + DB (idx / 4) .. + DB - 1, and the pairs are spread two slots apart behind that
-#ifndef MHIP_FWD_EARLY_STEP
-#define MHIP_FWD_EARLY_STEP 2
-#endif
   auto early_slot = [](int idx) {
-    return idx < 4 ? kSlotsS + DB + MHIP_FWD_EARLY_STEP * idx : kSlotsS + 3 * DB + (idx - 4);
+    return idx < 4 ? kSlotsS + DB + kEarlyStep * idx : kSlotsS + 3 * DB + (idx - 4);
   };
-  static_assert(kEarlyPairs <= 4 && kSlotsS + DB + MHIP_FWD_EARLY_STEP * (kEarlyPairs - 1) < kSlotsS + kSlotsO,
+  static_assert(kEarlyPairs <= 4 && kSlotsS + DB + kEarlyStep * (kEarlyPairs - 1) < kSlotsS + kSlotsO,
                 "the early pairs have to fit behind the O^T slots of k-step 0");
   auto sm_tile = [&]() {
 #pragma unroll
