@@ -83,26 +83,6 @@ def generated_ring_step(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False,
 '''
 
 
-def mfma_ceiling(torch, N, dev, cus):
-    """TFLOP/s and shader clock of a register-only loop of the bf16 MFMA (mhip_probe_mfma_ceiling), with constant
-    and with pseudo-random operands: what the power management of this box lets the matrix pipes sustain."""
-    sink = torch.empty(cus * 256, dtype=torch.float32, device=dev)
-    cyc = torch.zeros(1, dtype=torch.int64, device=dev)
-    out = {}
-    for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
-        iters = 40000                                  # x 32 MFMAs per wavefront: about 25 ms
-        for n in (iters // 20, iters):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            N.check(N.lib().mhip_probe_mfma_ceiling(N.ptr(sink), N.ptr(cyc), cus, n, rnd, N.stream_of(sink)), "probe")
-            e1.record()
-            torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1)
-        flops = cus * 4.0 * iters * 32 * 32768.0
-        out[name] = {"tflops": round(flops / ms / 1e9, 1), "clock_mhz": round(cyc.item() / ms / 1e3)}
-    return out
-
-
 def operand_dependence(torch, M, dev, shape, scale):
     """The headline block kernel (one chunk, 4096 x 4096) on operands that toggle few bits: all zeros, and small
     integers.  Same kernel, same instruction stream, same number of MFMAs; only the switching activity of the
@@ -226,7 +206,7 @@ def main() -> int:
                     help="seconds of back-to-back steps for the `sustained` figure (0 = skip)")
     ap.add_argument("--no-variants", action="store_true",
                     help="skip everything after the headline step: the short timings of the causal, backward and "
-                         "fp8 block kernels, the MFMA ceiling probe and the low-toggle operand runs")
+                         "fp8 block kernels and the low-toggle operand runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one rank's step on ONE GPU (the ring is emulated by local buffer rotation); "
@@ -478,7 +458,6 @@ def main() -> int:
     }
     result["sustained"] = sustained
     if variants is not None:
-        result["mfma_ceiling"] = mfma_ceiling(torch, M._native, dev, props.multi_processor_count)
         result["forward_kernel_on_low_toggle_operands"] = operand_dependence(torch, M, dev, (B, Sq, H, D), scale)
         result["other_kernels"] = variants
     if args.cpu_heads > 0:

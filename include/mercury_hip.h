@@ -45,6 +45,10 @@ extern "C" {
 #define MHIP_MASK_NONE    0
 #define MHIP_MASK_CAUSAL  1   /* query i sees key j iff j <= i + (Sc - Sq) (bottom-right) */
 
+/* Bumped whenever an entry point's argument list changes (a caller built against another value must not call).
+ * 3: the three descales of mhip_attn_fwd_block are device pointers; mhip_attn_bwd_block takes five stride triples. */
+#define MHIP_ABI_VERSION 3
+int         mhip_abi_version(void);   /* the MHIP_ABI_VERSION the library was built with */
 int         mhip_version(void);
 const char* mhip_error_string(int code);
 
@@ -53,8 +57,11 @@ const char* mhip_error_string(int code);
  * Replaces flash_attn.flash_attn_interface._flash_attn_forward as called at
  * utils/flash_attn_dsl.py:159-176 (dropout_p = 0, softcap = 0, no alibi, window (-1,-1)).
  * out has q's element type for MHIP_BF16 and is bf16 for MHIP_E4M3.  Rows that see no key
- * get out = 0 and lse = -inf.  For MHIP_E4M3 the three descales are the per-tensor fp32
- * scales s (x ~ s * x_q); ignored for MHIP_BF16.
+ * get out = 0 and lse = -inf.  For MHIP_E4M3 the three descales point to the per-tensor fp32
+ * scales s (x ~ s * x_q) in DEVICE memory, one float each, read by the kernel when it runs (so
+ * they may be written by earlier work on the stream, and a captured graph uses the values present
+ * at replay); NULL means 1.  They must be positive and finite (not checked: the values never
+ * reach the host).  Ignored for MHIP_BF16.
  * Head dimension: MHIP_BF16 any multiple of 8 up to 128 (the kernel computes on 128 columns, on 64 for D <= 64;
  * the missing ones are zeros that exist only on chip -- no padded copy, no extra memory traffic -- and the K / V
  * span Sc * stride of one (batch, head) must stay below 2^30 bytes, MHIP_EUNSUPPORTED beyond); MHIP_E4M3 any
@@ -67,7 +74,7 @@ int mhip_attn_fwd_block(const void* q, const void* k, const void* v, void* out, 
                         int64_t v_sb, int64_t v_ss, int64_t v_sh,
                         int64_t o_sb, int64_t o_ss, int64_t o_sh,
                         float softmax_scale, int mask, int dtype,
-                        float q_descale, float k_descale, float v_descale,
+                        const float* q_descale, const float* k_descale, const float* v_descale,
                         void* stream);
 
 /*
@@ -216,17 +223,6 @@ int mhip_unpack(const float* buf, void* out, float* lse, int B, int Sq, int Hq, 
  * dst = (acc ? acc : 0) + float(block), n elements, block in bf16; dst may alias acc.
  */
 int mhip_grad_accumulate(const float* acc, const void* block, float* dst, int64_t n, void* stream);
-
-/*
- * Measurement aid, no counterpart in the reference: a register-only loop of v_mfma_f32_32x32x16_bf16 (the
- * instruction of the bf16 block kernels), `workgroups` workgroups of four wavefronts, `iters` x 32 MFMAs per
- * wavefront, with operands that are constant (random_operands == 0) or pseudo-random bf16 values.  sink:
- * workgroups * 256 floats, cycles: one 64-bit count of shader clocks spent in the loop by the first
- * wavefront.  FLOP = workgroups * 4 * iters * 32 * 32768; bench.py times it to report the matrix-pipe ceiling
- * the power management of the box allows, next to the attention kernels' figures.
- */
-int mhip_probe_mfma_ceiling(float* sink, long long* cycles, int workgroups, int iters, int random_operands,
-                            void* stream);
 
 #ifdef __cplusplus
 }

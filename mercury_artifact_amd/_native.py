@@ -12,9 +12,10 @@ from typing import Optional
 
 import torch
 
-# MERCURY_HIP_LIB points at another build of the same library (e.g. one compiled with other tuning macros).
+# MERCURY_HIP_LIB is a deployment option: the path of the built library when it is not kept next to the package.
 LIB_PATH = os.environ.get("MERCURY_HIP_LIB") or os.path.join(
     os.path.dirname(os.path.abspath(__file__)), "csrc", "libmercury_hip.so")
+ABI_VERSION = 3      # MHIP_ABI_VERSION of include/mercury_hip.h the signatures below were written against
 
 MHIP_BF16, MHIP_E4M3, MHIP_F32 = 0, 1, 2
 MASK_NONE, MASK_CAUSAL = 0, 1
@@ -24,8 +25,9 @@ _lib = None
 _I, _L, _F, _P = c_int, c_int64, c_float, c_void_p
 _SIGNATURES = {
     "mhip_version": (c_int, []),
+    "mhip_abi_version": (c_int, []),
     "mhip_error_string": (ctypes.c_char_p, [_I]),
-    "mhip_attn_fwd_block": (c_int, [_P] * 5 + [_I] * 6 + [_L] * 12 + [_F, _I, _I, _F, _F, _F, _P]),
+    "mhip_attn_fwd_block": (c_int, [_P] * 5 + [_I] * 6 + [_L] * 12 + [_F, _I, _I, _P, _P, _P, _P]),
     "mhip_attn_bwd_workspace_bytes": (c_int64, [_I] * 6),
     "mhip_attn_bwd_block": (c_int, [_P] * 10 + [_I] * 6 + [_L] * 15 + [_F, _I, _I, _P, _P]),
     "mhip_attn_bwd_block_noalloc": (c_int, [_P] * 10 + [_I] * 6 + [_L] * 15 + [_F, _I, _I, _P]),
@@ -37,7 +39,6 @@ _SIGNATURES = {
     "mhip_unpack": (c_int, [_P] * 3 + [_I] * 4 + [_P]),
     "mhip_grad_accumulate": (c_int, [_P] * 3 + [_L, _P]),
     "mhip_quantize_e4m3": (c_int, [_P, _I, _L, _P, _P, _P, _P]),
-    "mhip_probe_mfma_ceiling": (c_int, [_P, _P, _I, _I, _I, _P]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 
@@ -50,6 +51,14 @@ def lib() -> ctypes.CDLL:
                 f"{LIB_PATH} is missing: build it with `python -m mercury_artifact_amd.csrc.build` "
                 "(hipcc, gfx950). There is no fallback implementation.")
         handle = ctypes.CDLL(LIB_PATH)
+        try:
+            handle.mhip_abi_version.restype = c_int
+            built = handle.mhip_abi_version()
+        except AttributeError:
+            built = None
+        if built != ABI_VERSION:
+            raise RuntimeError(f"{LIB_PATH} was built with ABI version {built}, this package calls version "
+                               f"{ABI_VERSION}: rebuild it with `python -m mercury_artifact_amd.csrc.build`")
         for name, (res, args) in _SIGNATURES.items():
             fn = getattr(handle, name)
             fn.restype = res

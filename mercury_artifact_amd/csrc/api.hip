@@ -8,12 +8,13 @@ int attn_fwd_bf16(const void* q, const void* k, const void* v, void* out, float*
                   const int64_t* strides, float scale, int mask, hipStream_t stream);
 int attn_fwd_fp8(const void* q, const void* k, const void* v, void* out, float* lse,
                  int B, int Sq, int Sc, int Hq, int Hkv, int D, const int64_t* strides, float scale, int mask,
-                 float q_descale, float k_descale, float v_descale, hipStream_t stream);
+                 const float* q_descale, const float* k_descale, const float* v_descale, hipStream_t stream);
 }  // namespace mhip
 
 using namespace mhip;
 
 extern "C" int mhip_version(void) { return 1; }
+extern "C" int mhip_abi_version(void) { return MHIP_ABI_VERSION; }
 
 extern "C" const char* mhip_error_string(int code) {
   switch (code) {
@@ -41,7 +42,7 @@ extern "C" int mhip_attn_fwd_block(const void* q, const void* k, const void* v, 
                                    int64_t v_sb, int64_t v_ss, int64_t v_sh,
                                    int64_t o_sb, int64_t o_ss, int64_t o_sh,
                                    float softmax_scale, int mask, int dtype,
-                                   float q_descale, float k_descale, float v_descale,
+                                   const float* q_descale, const float* k_descale, const float* v_descale,
                                    void* stream) {
   if (B < 0 || Sq < 0 || Sc < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return MHIP_EINVAL;
   if (!(softmax_scale > 0.f) || !(softmax_scale < INFINITY)) return MHIP_EINVAL;
@@ -68,7 +69,9 @@ extern "C" int mhip_attn_fwd_block(const void* q, const void* k, const void* v, 
   if (D < 128 && kv_span >= (int64_t(1) << 30)) return MHIP_EUNSUPPORTED;
   const int64_t strides[12] = {q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, v_sb, v_ss, v_sh, o_sb, o_ss, o_sh};
   if (fp8) {
-    if (!(q_descale > 0.f) || !(k_descale > 0.f) || !(v_descale > 0.f)) return MHIP_EINVAL;
+    if ((reinterpret_cast<uintptr_t>(q_descale) | reinterpret_cast<uintptr_t>(k_descale) |
+         reinterpret_cast<uintptr_t>(v_descale)) & 3u)
+      return MHIP_EALIGN;
     return attn_fwd_fp8(q, k, v, out, lse, B, Sq, Sc, Hq, Hkv, D, strides, softmax_scale, mask,
                         q_descale, k_descale, v_descale, st);
   }

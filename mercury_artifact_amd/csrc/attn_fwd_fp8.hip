@@ -44,9 +44,8 @@ struct Fp8Params {
   int B, Sq, Sc, Hq, Hkv, group;
   int D;             // head dimension of the tensors, a multiple of 16 up to kD; columns D .. kD-1 are zeros on chip
   int64_t q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, v_sb, v_ss, v_sh, o_sb, o_ss, o_sh;
-  float scale_eff;       // softmax_scale * q_descale * k_descale: natural-log scale of the integer-like dot
-  float scale_log2;      // scale_eff * log2(e)
-  float out_mul;         // v_descale
+  float scale;           // softmax scale
+  const float* q_descale; const float* k_descale; const float* v_descale;   // device scalars, NULL = 1
   int nq_tiles, total, per_xcd, heads_per_xcd;
 };
 
@@ -58,6 +57,14 @@ __device__ __forceinline__ constexpr int swz8(int row) { return (((row >> 1) & 3
 template <bool CAUSAL>
 __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Params p) {
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kStages * kTileBytes];
+
+  // The per-tensor descales are read from device memory here (one scalar load each), so a step whose operands are
+  // re-quantised every time needs no device-to-host copy and a captured graph sees the values of the replay.
+  const float qd = p.q_descale ? *p.q_descale : 1.f;
+  const float kd = p.k_descale ? *p.k_descale : 1.f;
+  const float out_mul = p.v_descale ? *p.v_descale : 1.f;
+  const float scale_eff = p.scale * qd * kd;      // natural-log scale of the integer-like dot
+  const float scale_log2 = scale_eff * kLog2e;
 
   // Workgroup i runs on XCD i % 8: every XCD gets a contiguous range of (batch, head) pairs, so the
   // workgroups that share a K/V head share an L2.  Causal launches run the longest Q tiles first,
@@ -247,10 +254,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
 #pragma unroll
       for (int j = 0; j < 16; ++j) mx = fmaxf(mx, s[mb][j]);
     mx = pair_max(mx);
-    const bool grow = (mx - m_ref) * p.scale_log2 > kRescaleSlack;
+    const bool grow = (mx - m_ref) * scale_log2 > kRescaleSlack;
     if (__builtin_amdgcn_ballot_w64(grow) != 0) {
       const float m_new = grow ? mx : m_ref;
-      const float alpha = (m_new == -INFINITY) ? 1.f : fast_exp2((m_ref - m_new) * p.scale_log2);
+      const float alpha = (m_new == -INFINITY) ? 1.f : fast_exp2((m_ref - m_new) * scale_log2);
       m_ref = m_new;
       l_run *= alpha;
 #pragma unroll
@@ -258,13 +265,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
 #pragma unroll
         for (int j = 0; j < 16; ++j) o_acc[db][j] *= alpha;
     }
-    const float msc = (m_ref == -INFINITY) ? 0.f : m_ref * p.scale_log2 - kPShift;   // exponent of 2^7 P
+    const float msc = (m_ref == -INFINITY) ? 0.f : m_ref * scale_log2 - kPShift;   // exponent of 2^7 P
     float rs = 0.f;
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) {
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
-        const float e = fast_exp2(__builtin_fmaf(s[mb][j], p.scale_log2, -msc));
+        const float e = fast_exp2(__builtin_fmaf(s[mb][j], scale_log2, -msc));
         rs += e;
         s[mb][j] = e;
       }
@@ -294,9 +301,9 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
 
   // ---- epilogue ---------------------------------------------------------------------------------------------
   const float l_tot = pair_sum(l_run);
-  const float inv = l_tot > 0.f ? p.out_mul / l_tot : 0.f;           // the two factors 2^7 cancel
+  const float inv = l_tot > 0.f ? out_mul / l_tot : 0.f;           // the two factors 2^7 cancel
   if (hf == 0 && my_q < p.Sq) {
-    const float lse = l_tot > 0.f ? m_ref * p.scale_eff + (fast_log2(l_tot) - kPShift) * kLn2 : -INFINITY;
+    const float lse = l_tot > 0.f ? m_ref * scale_eff + (fast_log2(l_tot) - kPShift) * kLn2 : -INFINITY;
     p.lse[((int64_t)b * p.Hq + hq) * p.Sq + my_q] = lse;
   }
   __syncthreads();
@@ -330,7 +337,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
 
 int attn_fwd_fp8(const void* q, const void* k, const void* v, void* out, float* lse,
                  int B, int Sq, int Sc, int Hq, int Hkv, int D, const int64_t* st, float scale, int mask,
-                 float q_descale, float k_descale, float v_descale, hipStream_t stream) {
+                 const float* q_descale, const float* k_descale, const float* v_descale, hipStream_t stream) {
   Fp8Params p;
   p.q = static_cast<const uint8_t*>(q); p.k = static_cast<const uint8_t*>(k); p.v = static_cast<const uint8_t*>(v);
   p.out = static_cast<uint16_t*>(out); p.lse = lse;
@@ -340,9 +347,8 @@ int attn_fwd_fp8(const void* q, const void* k, const void* v, void* out, float* 
   p.k_sb = st[3]; p.k_ss = st[4]; p.k_sh = st[5];
   p.v_sb = st[6]; p.v_ss = st[7]; p.v_sh = st[8];
   p.o_sb = st[9]; p.o_ss = st[10]; p.o_sh = st[11];
-  p.scale_eff = scale * q_descale * k_descale;
-  p.scale_log2 = p.scale_eff * kLog2e;
-  p.out_mul = v_descale;
+  p.scale = scale;
+  p.q_descale = q_descale; p.k_descale = k_descale; p.v_descale = v_descale;
   p.nq_tiles = (Sq + kBM - 1) / kBM;
   p.total = B * Hq * p.nq_tiles;
   p.per_xcd = (p.total + 7) / 8;

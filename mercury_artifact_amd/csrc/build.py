@@ -10,7 +10,7 @@ import sys
 from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = ["api.hip", "attn_fwd.hip", "attn_fwd_fp8.hip", "attn_bwd.hip", "lse_merge.hip", "quantize.hip", "probe.hip"]
+SOURCES = ["api.hip", "attn_fwd.hip", "attn_fwd_fp8.hip", "attn_bwd.hip", "lse_merge.hip", "quantize.hip"]
 LIB = os.path.join(HERE, "libmercury_hip.so")
 # -packed-fp32-ops off: keep the compiler from forming v_pk_{add,mul,fma}_f32.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall",

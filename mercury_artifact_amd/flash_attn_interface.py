@@ -44,25 +44,26 @@ def _check_block_inputs(q, k, v, dropout_p, window_size_left, window_size_right,
         raise RuntimeError("number of query heads must be a multiple of the number of KV heads")
 
 
-def _host_scalar(t) -> float:
-    """The value of a descale as a host float.  The C ABI takes the three descales by value, and a descale
-    usually is a 0-dim tensor on the device (quantize_e4m3 returns one): reading it costs a device-to-host
-    synchronisation, so the value is read once per tensor object and kept on it (keyed by the tensor's version
-    counter, so an in-place update is seen).  A step that reuses its descale tensors then synchronises three
-    times in all instead of three times per block, and can be captured in a HIP graph after one eager run."""
+_DESCALE_CONSTANTS = {}
+
+
+def _descale_pointer(t, device):
+    """A descale as the kernel wants it: one float32 in device memory, read by the kernel when it runs.  A tensor is
+    passed as it is (no copy to the host, no synchronisation: a step that re-quantises its operands every time, or
+    a captured graph whose scales are rewritten between replays, sees the current value); a Python number becomes
+    a one-element device tensor, made once per (device, value) and kept."""
     if t is None:
-        return 1.0
-    if not isinstance(t, torch.Tensor):
-        return float(t)
-    cached = getattr(t, "_mhip_host_value", None)
-    if cached is not None and cached[0] == t._version:
-        return cached[1]
-    value = float(t)
-    try:
-        t._mhip_host_value = (t._version, value)
-    except AttributeError:
-        pass
-    return value
+        return None
+    if isinstance(t, torch.Tensor):
+        if t.numel() != 1 or t.dtype != torch.float32:
+            raise RuntimeError("a descale must be a float32 tensor with one element (per-tensor scale)")
+        return t
+    key = (str(device), float(t))
+    cached = _DESCALE_CONSTANTS.get(key)
+    if cached is None:
+        cached = torch.tensor([float(t)], dtype=torch.float32, device=device)
+        _DESCALE_CONSTANTS[key] = cached
+    return cached
 
 
 def attn_fwd_block(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float,
@@ -75,7 +76,7 @@ def attn_fwd_block(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_sc
     missing ones with zeros on chip, which changes neither the scores nor the columns that exist);
     float8_e4m3fn: any multiple of 16 up to 128, in the same way."""
     _check_block_inputs(q, k, v, 0, -1, -1, 0.0, None)
-    N.require_cuda(out, lse, q_descale, k_descale, v_descale)
+    N.require_cuda(out, lse)
     B, Sq, Hq, D = q.shape
     _, Sc, Hkv, _ = k.shape
     if q.dtype == torch.bfloat16:
@@ -94,14 +95,15 @@ def attn_fwd_block(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_sc
         lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
     elif lse.shape != (B, Hq, Sq) or lse.dtype != torch.float32 or not lse.is_contiguous():
         raise RuntimeError("lse must be a contiguous float32 (B, Hq, Sq) tensor")
-    ds = [_host_scalar(t) for t in (q_descale, k_descale, v_descale)]
+    ds = [_descale_pointer(t, q.device) for t in (q_descale, k_descale, v_descale)]
+    N.require_cuda(*ds)
     with torch.cuda.device(q.device):
         code = N.lib().mhip_attn_fwd_block(
             N.ptr(q), N.ptr(k), N.ptr(v), N.ptr(out), N.ptr(lse),
             B, Sq, Sc, Hq, Hkv, D,
             *_strides3(q), *_strides3(k), *_strides3(v), *_strides3(out),
             float(softmax_scale), N.MASK_CAUSAL if causal else N.MASK_NONE, dt,
-            ds[0], ds[1], ds[2], N.stream_of(q))
+            N.ptr(ds[0]), N.ptr(ds[1]), N.ptr(ds[2]), N.stream_of(q))
     N.check(code, "mhip_attn_fwd_block")
     return out, lse
 

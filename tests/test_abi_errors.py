@@ -16,7 +16,7 @@ def lib():
 
 
 def _fwd(lib, q=P, k=P, v=P, out=P, lse=P, B=1, Sq=64, Sc=64, Hq=2, Hkv=2, D=128,
-         strides=None, scale=0.1, mask=0, dtype=0, descales=(1.0, 1.0, 1.0)):
+         strides=None, scale=0.1, mask=0, dtype=0, descales=(None, None, None)):
     if strides is None:
         strides = [Sq * Hq * D, Hq * D, D, Sc * Hkv * D, Hkv * D, D, Sc * Hkv * D, Hkv * D, D, Sq * Hq * D, Hq * D, D]
     return lib.mhip_attn_fwd_block(q, k, v, out, lse, B, Sq, Sc, Hq, Hkv, D, *strides, scale, mask, dtype,
@@ -46,7 +46,7 @@ def test_forward_rejects(lib):
     big = 1 << 20                               # rows 2 MiB apart: 2048 of them span 4 GiB
     assert _fwd(lib, Sc=2048, strides=[64 * 256, 256, 128, 2048 * big, big, 128, 2048 * big, big, 128,
                                        64 * 256, 256, 128]) == EUNSUPPORTED
-    assert _fwd(lib, dtype=1, descales=(1.0, 0.0, 1.0)) == EINVAL
+    assert _fwd(lib, dtype=1, descales=(P, P + 2, P)) == EALIGN    # descales are pointers to device floats
     # nothing to do: accepted without touching the pointers
     assert _fwd(lib, B=0) == OK
     assert _fwd(lib, Sq=0) == OK

@@ -141,8 +141,9 @@ def test_search_harness_bench_program_allocates_execs_and_times(lazy, capsys):
 
 
 def test_graphed_fp8_step_matches_eager():
-    """The fp8 step takes its three descales as device scalars; their host values are read once per tensor, so
-    the step can be captured after the warm-up runs and replays bit-identically."""
+    """The fp8 step takes its three descales as device scalars that the kernel reads when it runs: the step is
+    captured without any device-to-host copy, replays bit-identically, and a replay after the scales were rewritten
+    in place (the normal case of re-quantising every step) uses the new values, as the eager step does."""
     import mercury_artifact_amd as M
 
     B, S, H, D, W, rank = 1, 256, 2, 128, 2, 1
@@ -169,9 +170,39 @@ def test_graphed_fp8_step_matches_eager():
         graphed.replay()
         torch.cuda.synchronize()
         assert torch.equal(o, eo) and torch.equal(lse, el), it
-    # an in-place change of a descale is seen by the next eager call (the cache is keyed by the version counter)
-    before = o.clone()
+    # descales rewritten in place between replays: by a torch op, and through the raw pointer (a write no version
+    # counter sees); eager call and replay both read the value that is in memory when the kernel runs
+    before_o, before_l = o.clone(), lse.clone()
     sv.mul_(2.0)
     step()
     torch.cuda.synchronize()
-    assert torch.allclose(o.float(), 2.0 * before.float(), rtol=2 ** -7, atol=1e-6)
+    assert torch.allclose(o.float(), 2.0 * before_o.float(), rtol=2 ** -7, atol=1e-6) and torch.equal(lse, before_l)
+    o.zero_()
+    graphed.replay()
+    torch.cuda.synchronize()
+    assert torch.allclose(o.float(), 2.0 * before_o.float(), rtol=2 ** -7, atol=1e-6)
+    sq.mul_(0.5)
+    step()
+    torch.cuda.synchronize()
+    eo, el = o.clone(), lse.clone()
+    assert not torch.equal(el, before_l)
+    o.zero_()
+    lse.zero_()
+    graphed.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(o, eo) and torch.equal(lse, el)
+    import ctypes
+    half = (ctypes.c_float * 1)(float(sk) * 0.5)
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+    assert hip.hipMemcpy(sk.data_ptr(), ctypes.addressof(half), 4, 1) == 0        # 1 = host to device
+    torch.cuda.synchronize()
+    step()
+    torch.cuda.synchronize()
+    eo2, el2 = o.clone(), lse.clone()
+    assert not torch.equal(el2, el)
+    o.zero_()
+    lse.zero_()
+    graphed.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(o, eo2) and torch.equal(lse, el2)
