@@ -19,8 +19,8 @@ from .ring import (flash_attn_backward, flash_attn_expose_reduce, flash_attn_exp
                    flash_attn_pack_kv,
                    flash_attn_pack_split_kv, fp8_pack_split_kv, gqa_pack_kv, quantize_e4m3,
                    zigzag_causal_pack_kv)
-from .schedule import (LocalRing, double_ring_order, get_src_dst_ranks, n_dim_to_one_dim,
-                       one_dim_to_n_dim, reduce_buffer_route, ring_divide_order, shift_tuple_element, single_ring_order,
+from .schedule import (LocalMesh, LocalRing, debug_print, double_ring_order, get_device_group, get_src_dst_ranks, local_peers,
+                       n_dim_to_one_dim, one_dim_to_n_dim, reduce_buffer_route, ring_divide_order, shift_tuple_element, single_ring_order,
                        zigzag_blocks, zigzag_step)
 
 __version__ = "0.1.0"
@@ -48,4 +48,6 @@ def namespace(lazy_merge: bool = False) -> dict:
         "n_dim_to_one_dim": n_dim_to_one_dim,
         "shift_tuple_element": shift_tuple_element,
         "get_src_dst_ranks": get_src_dst_ranks,
+        "get_device_group": get_device_group,
+        "debug_print": debug_print,
     }

@@ -13,6 +13,7 @@ from typing import Optional, Sequence, Tuple
 import torch
 
 from . import _native as N
+from .schedule import LocalGroup
 
 __all__ = ["get_default_args", "update_out_and_lse", "_update_out_and_lse", "flash_reduce",
            "pack_block", "unpack_into", "merge_into", "merge_many", "grad_accumulate", "update_out_and_lse_collective", "add_collective",
@@ -184,20 +185,6 @@ def flash_reduce(lhs: torch.Tensor, rhs: torch.Tensor) -> torch.Tensor:
     return dst
 
 
-class LocalGroup:
-    """Single-GPU stand-in for the process group of a collective: ``peers`` are the operands of all ranks
-    of the group as they are when the collective starts, ``rank`` the position of the calling rank."""
-
-    def __init__(self, peers: Sequence[torch.Tensor], rank: int = 0):
-        if not 0 <= rank < len(peers):
-            raise ValueError("rank outside the group")
-        self.peers = list(peers)
-        self.rank = rank
-
-    def size(self) -> int:
-        return len(self.peers)
-
-
 def _is_collective(op, name: str) -> bool:
     return op == name or getattr(op, "__name__", None) == name
 
@@ -216,12 +203,12 @@ def update_out_and_lse_collective(tensor: torch.Tensor, op, group: LocalGroup, d
     ``group`` the tree-attention way (MAX of the lse, SUM of ``out * d`` and ``d``) and write the merged
     value into ``tensor`` in place.  ``op`` is ``dist.all_reduce`` or ``dist.reduce`` (the function or its
     name); with ``reduce`` only rank ``dst`` receives the result.  The per-rank arithmetic runs in two
-    kernels (``mhip_tree_merge``); the collectives themselves are replayed over ``group.peers``: one MAX
+    kernels (``mhip_tree_merge``); the collectives themselves are replayed over the operands of the group's ranks: one MAX
     over the lse columns and ONE SUM over the packed ``(out * d | d)`` terms."""
     reduce_to_one = _is_collective(op, "reduce")
     if not (reduce_to_one or _is_collective(op, "all_reduce")):
         raise RuntimeError("Unsupported collective op")
-    peers = [p.contiguous() for p in group.peers]
+    peers = [p.contiguous() for p in group.operands(tensor)]
     N.require_cuda(tensor, *peers)
     for p in peers:
         if p.shape != tensor.shape or p.dtype != torch.float32:
@@ -234,7 +221,7 @@ def update_out_and_lse_collective(tensor: torch.Tensor, op, group: LocalGroup, d
         term = torch.empty_like(p)
         _tree_merge(p, row_max, term, finish=False)
         total = term if total is None else total.add_(term)   # the SUM all-reduce
-    if reduce_to_one and dst is not None and dst != group.rank:
+    if reduce_to_one and dst is not None and dst != group.ranks[group.rank]:      # dst is a global rank
         return
     out = tensor if tensor.is_contiguous() else torch.empty_like(total)
     _tree_merge(total, row_max, out, finish=True)
@@ -248,7 +235,7 @@ def add_collective(tensor: torch.Tensor, op, group: LocalGroup, dst: Optional[in
     if not _is_collective(op, "all_reduce"):
         raise ValueError("not support other op than all reduce")
     total = None
-    for p in group.peers:
+    for p in group.operands(tensor):
         total = p.to(torch.float32, copy=True) if total is None else total.add_(p)
     tensor.copy_(total)
 

@@ -7,13 +7,16 @@ hands the emulated rank the chunk it would have received -- buffer rotation in p
 """
 from __future__ import annotations
 
+import contextlib
+import queue
+import threading
 from functools import lru_cache
-from typing import List, Optional, Sequence, Tuple
+from typing import Callable, List, Optional, Sequence, Tuple
 
 import torch
 
 __all__ = ["one_dim_to_n_dim", "n_dim_to_one_dim", "shift_tuple_element", "get_src_dst_ranks",
-           "LocalRing", "single_ring_order", "double_ring_order", "ring_divide_order",
+           "get_device_group", "debug_print", "LocalGroup", "local_peers", "LocalMesh", "LocalRing", "single_ring_order", "double_ring_order", "ring_divide_order",
            "zigzag_blocks", "zigzag_step"]
 
 
@@ -60,6 +63,94 @@ def get_src_dst_ranks(indices: Tuple[int, ...], mesh_shape: Tuple[int, ...],
         dst = shift_tuple_element(dst, dim, step, mesh_shape[dim])
         step = mesh_shape[dim]
     return n_dim_to_one_dim(src, tuple(mesh_shape)), n_dim_to_one_dim(dst, tuple(mesh_shape))
+
+
+# ------------------------------------------------------------------------------------------------
+# communication groups of a collective, and their single-GPU stand-in
+# ------------------------------------------------------------------------------------------------
+_PEER_SOURCE: List[Optional[Callable[[int], torch.Tensor]]] = [None]
+_ACTIVE_MESH: List[Optional["LocalMesh"]] = [None]
+
+
+@contextlib.contextmanager
+def local_peers(source: Callable[[int], torch.Tensor]):
+    """While the block runs, the groups ``get_device_group`` hands out take the operands of the ranks that are not
+    the calling one from ``source(rank)``: on one GPU there is no peer to reduce with, so whoever emulates a
+    mesh says what the other ranks would contribute (their partial results as they are when the collective
+    starts)."""
+    before = _PEER_SOURCE[0]
+    _PEER_SOURCE[0] = source
+    try:
+        yield
+    finally:
+        _PEER_SOURCE[0] = before
+
+
+class LocalGroup:
+    """Single-GPU stand-in for the process group of a collective.  Either ``peers`` -- the operands of all ranks
+    of the group as they are when the collective starts, ``rank`` the position of the calling rank among them --
+    or, as ``get_device_group`` builds it, the global ``ranks`` of the group: the operands of the other ranks
+    are then asked of the source installed by ``local_peers`` when the collective runs."""
+
+    def __init__(self, peers: Optional[Sequence[torch.Tensor]] = None, rank: int = 0,
+                 ranks: Optional[Sequence[int]] = None):
+        if peers is None and ranks is None:
+            raise ValueError("a group needs the operands of its ranks or their rank numbers")
+        n = len(peers) if peers is not None else len(ranks)
+        if not 0 <= rank < n:
+            raise ValueError("rank outside the group")
+        self.peers = list(peers) if peers is not None else None
+        self.ranks = tuple(ranks) if ranks is not None else tuple(range(n))
+        self.rank = rank
+
+    def size(self) -> int:
+        return len(self.ranks)
+
+    def operands(self, mine: torch.Tensor) -> List[torch.Tensor]:
+        """Operands of all ranks of the group, the calling rank's being ``mine``."""
+        if self.peers is not None:
+            return list(self.peers)
+        if _ACTIVE_MESH[0] is not None:
+            return _ACTIVE_MESH[0]._gather(self.ranks, mine)
+        source = _PEER_SOURCE[0]
+        if source is None and len(self.ranks) > 1:
+            raise RuntimeError("this group was built by get_device_group on one GPU: run the collective inside "
+                               "`with local_peers(source):` so that the other ranks' operands are known")
+        return [mine if i == self.rank else source(r) for i, r in enumerate(self.ranks)]
+
+
+@lru_cache(maxsize=None)
+def get_device_group(indices: Tuple[int, ...], mesh_shape: Tuple[int, ...], dims: Tuple[int, ...], debug: bool = False):
+    """Communication group of the rank at mesh coordinates ``indices`` over the mesh dimensions ``dims``
+    (mercury/backend/pytorch/utils.py:114-169): all ranks whose coordinates agree with ``indices`` outside
+    ``dims``.  ``debug=True`` returns their sorted rank numbers, as the reference does; otherwise the reference
+    returns a ``dist.new_group`` of them, and this build, which runs one rank per process on one GPU, a
+    ``LocalGroup`` over the same ranks (see ``local_peers``)."""
+    indices, mesh_shape, dims = tuple(indices), tuple(mesh_shape), tuple(dims)
+    for dim in dims:
+        if dim < 0 or dim >= len(mesh_shape):
+            raise ValueError(f"Invalid dimension index: {dim}, mesh shape: {mesh_shape}")
+    members = [indices]
+    for dim in dims:
+        members = [m[:dim] + (i,) + m[dim + 1:] for m in members for i in range(mesh_shape[dim])]
+    ranks = tuple(sorted({n_dim_to_one_dim(m, mesh_shape) for m in members}))
+    if debug:
+        return ranks
+    return LocalGroup(ranks=ranks, rank=ranks.index(n_dim_to_one_dim(indices, mesh_shape)))
+
+
+def debug_print(*args) -> None:
+    """``print`` with the rank in front, one rank after the other (mercury/backend/pytorch/utils.py:108-112);
+    without an initialised process group there is one rank and nothing to take turns with."""
+    import torch.distributed as dist
+
+    if not (dist.is_available() and dist.is_initialized()):
+        print("[Rank 0]", *args)
+        return
+    for rank in range(dist.get_world_size()):
+        if rank == dist.get_rank():
+            print(f"[Rank {rank}]", *args)
+        dist.barrier()
 
 
 def reduce_buffer_route(mesh_shape: Sequence[int]) -> Tuple[List[List[int]], List[int]]:
@@ -215,3 +306,152 @@ class LocalRing:
             raise RuntimeError("wait called before commit")
         self._committed = False
         self._pending = False
+
+
+class LocalMesh:
+    """Every rank of a mesh as one thread of this process, all on the one GPU and on one stream: what a multi-rank
+    launch of a generated step function does, replayed where there is a single device.  ``run(fn)`` calls
+    ``fn(rank)`` in one thread per rank; inside, ``dist`` stands in for ``torch.distributed`` (``get_rank`` is the
+    thread's rank), ``SendRecv()`` gives an object with the reference's ``send_recv / commit / wait`` protocol
+    (mercury/backend/pytorch/utils.py:9-39) whose messages travel through per-pair mailboxes, and the groups of
+    ``get_device_group`` gather the operands of their ranks when a collective runs.  A message is a copy taken at
+    ``commit`` (as on a wire); since all threads enqueue on one stream, a receiver's copy is ordered behind the
+    kernels that produced the message.  Nothing blocks for longer than ``timeout`` seconds: a rank that waits for
+    a message nobody sends raises instead of hanging."""
+
+    def __init__(self, mesh_shape: Sequence[int], timeout: float = 60.0):
+        self.mesh_shape = tuple(int(x) for x in mesh_shape)
+        self.world = 1
+        for m in self.mesh_shape:
+            self.world *= m
+        self.timeout = timeout
+        self._tls = threading.local()
+        self._mail = {}
+        self._lock = threading.Lock()
+        self._gathers = {}
+        self._world_barrier = threading.Barrier(self.world)
+        mesh = self
+
+        class _Dist:
+            """The few names of torch.distributed that generated code touches."""
+
+            @staticmethod
+            def get_rank() -> int:
+                return mesh.rank()
+
+            @staticmethod
+            def get_world_size() -> int:
+                return mesh.world
+
+            @staticmethod
+            def barrier() -> None:
+                mesh._world_barrier.wait(mesh.timeout)
+
+            @staticmethod
+            def all_reduce(*args, **kwargs):
+                raise RuntimeError("collectives run inside update_out_and_lse_collective / add_collective")
+
+            @staticmethod
+            def reduce(*args, **kwargs):
+                raise RuntimeError("collectives run inside update_out_and_lse_collective / add_collective")
+
+        self.dist = _Dist
+
+    def rank(self) -> int:
+        return self._tls.rank
+
+    def _box(self, src: int, dst: int) -> "queue.Queue":
+        with self._lock:
+            return self._mail.setdefault((src, dst), queue.Queue())
+
+    def SendRecv(self) -> "_MeshSendRecv":
+        return _MeshSendRecv(self)
+
+    def _gather(self, ranks: Tuple[int, ...], mine: torch.Tensor) -> List[torch.Tensor]:
+        """Operands of all ranks of a group, each a copy taken when its rank arrived at the collective."""
+        with self._lock:
+            slot = self._gathers.get(ranks)
+            if slot is None:
+                slot = self._gathers[ranks] = {"barrier": threading.Barrier(len(ranks)), "parts": {}}
+        slot["parts"][self.rank()] = mine.clone()
+        slot["barrier"].wait(self.timeout)
+        parts = [slot["parts"][r] for r in ranks]
+        slot["barrier"].wait(self.timeout)          # everyone has read before the next collective writes
+        return parts
+
+    def run(self, fn: Callable[[int], object], ranks: Optional[Sequence[int]] = None) -> List[object]:
+        """``fn(rank)`` for every rank (or the given ones) at once; returns their results in rank order and
+        re-raises the first exception of any rank."""
+        ranks = list(range(self.world)) if ranks is None else list(ranks)
+        results = {}
+        errors = {}
+        device = torch.cuda.current_device() if torch.cuda.is_available() else None
+        stream = torch.cuda.current_stream() if torch.cuda.is_available() else None
+
+        def body(r):
+            self._tls.rank = r
+            try:
+                if device is not None:
+                    torch.cuda.set_device(device)
+                    with torch.cuda.stream(stream):
+                        results[r] = fn(r)
+                else:
+                    results[r] = fn(r)
+            except BaseException as exc:          # noqa: BLE001 -- handed to the caller below
+                errors[r] = exc
+                for slot in list(self._gathers.values()):
+                    slot["barrier"].abort()
+                self._world_barrier.abort()
+
+        if _ACTIVE_MESH[0] is not None:
+            raise RuntimeError("a LocalMesh is already running")
+        _ACTIVE_MESH[0] = self
+        try:
+            threads = [threading.Thread(target=body, args=(r,), daemon=True) for r in ranks]
+            for t in threads:
+                t.start()
+            for t in threads:
+                t.join()
+        finally:
+            _ACTIVE_MESH[0] = None
+        if errors:
+            first = min(errors)
+            real = [r for r in sorted(errors) if not isinstance(errors[r], threading.BrokenBarrierError)]
+            raise errors[real[0] if real else first]
+        return [results[r] for r in ranks]
+
+
+class _MeshSendRecv:
+    """``SendRecv`` of one rank of a ``LocalMesh``: same calls, same misuse errors as the reference's."""
+
+    def __init__(self, mesh: LocalMesh):
+        self._mesh = mesh
+        self._ops = []
+        self._committed = False
+
+    def send_recv(self, to_rank: int, from_rank: int, send_tensor: torch.Tensor,
+                  recv_tensor: Optional[torch.Tensor] = None) -> torch.Tensor:
+        res = torch.empty_like(send_tensor) if recv_tensor is None else recv_tensor
+        self._ops.append((to_rank, from_rank, send_tensor.contiguous(), res))
+        return res
+
+    def commit(self) -> None:
+        if self._committed:
+            raise RuntimeError("commit called twice")
+        me = self._mesh.rank()
+        for to_rank, _, send_tensor, _ in self._ops:
+            self._mesh._box(me, to_rank).put(send_tensor.clone())
+        self._committed = True
+
+    def wait(self) -> None:
+        if not self._committed:
+            raise RuntimeError("wait called before commit")
+        me = self._mesh.rank()
+        for _, from_rank, _, res in self._ops:
+            try:
+                got = self._mesh._box(from_rank, me).get(timeout=self._mesh.timeout)
+            except queue.Empty:
+                raise RuntimeError(f"rank {me} waited {self._mesh.timeout} s for a message from rank {from_rank}") from None
+            res.copy_(got)
+        self._committed = False
+        self._ops = []
