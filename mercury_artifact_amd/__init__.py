@@ -26,14 +26,15 @@ from .schedule import (LocalMesh, LocalRing, debug_print, double_ring_order, get
 __version__ = "0.1.0"
 
 
-def namespace(lazy_merge: bool = False) -> dict:
+def namespace(lazy_merge: bool = True) -> dict:
     """Names to place in the dict generated ring code is ``exec``-ed in (the reference fills it with
     ``from utils.flash_attn_dsl import *`` and ``from mercury.backend import *``).
 
-    ``lazy_merge=True`` binds ``update_out_and_lse`` to the recording variant of ``mercury_artifact_amd.lazy``:
-    unchanged generated code then folds all block results of a step in one pass when its epilogue runs,
-    instead of moving the fp32 accumulator once per chunk (same results to fp32 rounding; anything the lazy
-    handles are not asked by the generated epilogue falls back to the literal chain)."""
+    By default ``update_out_and_lse`` is the recording variant of ``mercury_artifact_amd.lazy``: unchanged
+    generated code then folds all block results of a step in one pass when its epilogue runs, instead of
+    moving the fp32 accumulator once per chunk (same results to fp32 rounding; anything the lazy handles are
+    not asked by the generated epilogue falls back to the literal chain).  ``lazy_merge=False`` binds the
+    literal merge of utils/flash_attn_dsl.py:51-71, one kernel per call."""
     return {
         "_flash_attn_forward": _flash_attn_forward,
         "_flash_attn_backward": _flash_attn_backward,

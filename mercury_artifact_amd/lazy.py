@@ -73,7 +73,75 @@ class _Pending:
         return self.chain
 
 
-class _Handle:
+def _real(x):
+    """Handles replaced by the tensors they stand for (inside lists and tuples too)."""
+    if isinstance(x, _TensorLike):
+        return x.materialize()
+    if isinstance(x, (list, tuple)):
+        return type(x)(_real(y) for y in x)
+    return x
+
+
+class _TensorLike:
+    """Behaves like the tensor ``materialize()`` returns for everything a subclass does not answer lazily:
+    attributes and methods, indexing, torch functions, and the operators Python looks up on the type
+    (arithmetic, comparisons, unary, in-place, ``len`` / ``iter`` / ``bool`` / ``float``)."""
+
+    def materialize(self) -> torch.Tensor:
+        raise NotImplementedError
+
+    def __getattr__(self, name):
+        return getattr(self.materialize(), name)
+
+    def __getitem__(self, item):
+        return self.materialize()[_real(item)]
+
+    def __setitem__(self, item, value):
+        self.materialize()[_real(item)] = _real(value)
+
+    @classmethod
+    def __torch_function__(cls, func, types, args=(), kwargs=None):
+        return func(*_real(args), **{k: _real(v) for k, v in (kwargs or {}).items()})
+
+    __hash__ = object.__hash__
+
+
+def _install_operators():
+    def binary(name):
+        def op(self, other):
+            return getattr(self.materialize(), name)(_real(other))
+        op.__name__ = name
+        return op
+
+    def inplace(name):
+        def op(self, other):
+            getattr(self.materialize(), name)(_real(other))
+            return self                      # the handle goes on standing for the tensor that was updated
+        op.__name__ = name
+        return op
+
+    def unary(name):
+        def op(self):
+            return getattr(self.materialize(), name)()
+        op.__name__ = name
+        return op
+
+    arithmetic = ["add", "sub", "mul", "truediv", "floordiv", "mod", "pow", "matmul", "and", "or", "xor",
+                  "lshift", "rshift"]
+    for base in arithmetic:
+        setattr(_TensorLike, f"__{base}__", binary(f"__{base}__"))
+        setattr(_TensorLike, f"__r{base}__", binary(f"__r{base}__"))
+        setattr(_TensorLike, f"__i{base}__", inplace(f"__i{base}__"))
+    for base in ["lt", "le", "gt", "ge", "eq", "ne"]:
+        setattr(_TensorLike, f"__{base}__", binary(f"__{base}__"))
+    for base in ["neg", "pos", "abs", "invert", "len", "iter", "bool", "float", "int", "index"]:
+        setattr(_TensorLike, f"__{base}__", unary(f"__{base}__"))
+
+
+_install_operators()
+
+
+class _Handle(_TensorLike):
     """Stands for one of the two accumulators; everything it is not asked lazily goes to the real tensor."""
 
     _which = 0
@@ -92,25 +160,6 @@ class _Handle:
     def device(self):
         return self._p.blocks[0][0].device
 
-    def __getattr__(self, name):
-        return getattr(self.materialize(), name)
-
-    def __getitem__(self, item):
-        return self.materialize()[item]
-
-    def __setitem__(self, item, value):
-        self.materialize()[item] = value
-
-    @classmethod
-    def __torch_function__(cls, func, types, args=(), kwargs=None):
-        def real(x):
-            if isinstance(x, _Handle):
-                return x.materialize()
-            if isinstance(x, (list, tuple)):
-                return type(x)(real(y) for y in x)
-            return x
-        return func(*real(args), **{k: real(v) for k, v in (kwargs or {}).items()})
-
 
 class LazyOut(_Handle):
     _which = 0
@@ -128,11 +177,11 @@ class LazyOut(_Handle):
         return self.materialize().to(*args, **kwargs)
 
 
-class _SqueezedLse:
+class _SqueezedLse(_TensorLike):
     """``_lse.squeeze(dim=-1)``: (B, Sq, Hq) in the reference; only ``transpose(1, 2)`` is answered lazily."""
 
     def __init__(self, pending: _Pending):
-        self._p = pending
+        object.__setattr__(self, "_p", pending)
 
     def materialize(self) -> torch.Tensor:
         return self._p.run_chain()[1].squeeze(dim=-1)
@@ -141,9 +190,6 @@ class _SqueezedLse:
         if sorted((dim0 % 3, dim1 % 3)) == [1, 2] and self._p.foldable():
             return self._p.fold()[1]
         return self.materialize().transpose(dim0, dim1)
-
-    def __getattr__(self, name):
-        return getattr(self.materialize(), name)
 
 
 class LazyLse(_Handle):

@@ -136,7 +136,7 @@ def test_generated_style_text_runs_in_the_namespace(text, name, rank):
     dev = [c.cuda() for c in kvs]
     ring = M.LocalRing((W,), rank, dev)
     namespace = {"torch": torch, "os": os, "dist": _Dist(rank), "WORLD": W, "SendRecv": lambda: ring}
-    namespace.update(M.namespace())
+    namespace.update(M.namespace(lazy_merge=False))
     exec(text, namespace)
     o = torch.empty(B, S // W, H, D, dtype=torch.bfloat16, device="cuda")
     lse = torch.empty(B, H, S // W, dtype=torch.float32, device="cuda")

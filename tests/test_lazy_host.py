@@ -165,3 +165,31 @@ def test_first_call_with_slice_raises_like_the_reference():
     outs, lses = _blocks(1, seed=7)
     with pytest.raises(RuntimeError, match="first update_out_and_lse should not pass slice_ args"):
         L.update_out_and_lse_lazy(None, None, outs[0], lses[0], slice_=(slice(None), slice(0, 4)))
+
+
+def test_operators_on_handles_act_on_the_real_tensors(cpu_merges):
+    """Python looks operators up on the type, not through __getattr__: arithmetic, comparisons, unary, in-place
+    operators, len() and torch functions on a handle (and on the squeezed LSE) all give what the literal
+    accumulators give."""
+    outs, lses = _blocks(3, seed=9)
+    h_out, h_lse = None, None
+    for bo, bl in zip(outs, lses):
+        h_out, h_lse = L.update_out_and_lse_lazy(h_out, h_lse, bo, bl)
+    ref_out, ref_lse = _reference(outs, lses)            # fp32 (B,S,H,D), (B,S,H,1)
+    assert torch.equal(h_out * 2.0, ref_out * 2.0)
+    assert torch.equal(2.0 * h_out, ref_out * 2.0)
+    assert torch.equal(-h_out, -ref_out)
+    assert torch.equal(h_out / h_out.abs().clamp_min(1.0), ref_out / ref_out.abs().clamp_min(1.0))
+    assert torch.equal(h_out - h_out, torch.zeros_like(ref_out))
+    assert bool(((h_lse > -1e30) == (ref_lse > -1e30)).all())
+    assert len(h_out) == ref_out.shape[0]
+    sq = h_lse.squeeze(dim=-1)
+    assert torch.equal(torch.transpose(sq, 1, 2), ref_lse.squeeze(-1).transpose(1, 2))      # a torch function on it
+    assert torch.equal(sq + 1.0, ref_lse.squeeze(-1) + 1.0)
+    assert torch.equal(sq[:, 2:5], ref_lse.squeeze(-1)[:, 2:5])
+    # in place: the handle goes on standing for the updated accumulator
+    same = h_out
+    h_out *= 0.5
+    assert h_out is same and torch.equal(h_out.materialize(), ref_out * 0.5)
+    assert torch.equal(h_out.to(torch.bfloat16), (ref_out * 0.5).to(torch.bfloat16))
+    assert cpu_merges.fold == 0
