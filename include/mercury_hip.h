@@ -50,6 +50,10 @@ extern "C" {
 #define MHIP_ABI_VERSION 3
 int         mhip_abi_version(void);   /* the MHIP_ABI_VERSION the library was built with */
 int         mhip_version(void);
+/* Optional: per-device set-up the entry points otherwise do on their first call on a device (today: the address
+ * of the scratch of mhip_attn_bwd_block_noalloc).  Cheap, idempotent, allocates nothing; MHIP_ERUNTIME if the
+ * runtime query fails.  Call it outside stream capture. */
+int         mhip_init(void);
 const char* mhip_error_string(int code);
 
 /*
@@ -84,7 +88,9 @@ int mhip_attn_fwd_block(const void* q, const void* k, const void* v, void* out, 
  * (B,Sc,Hkv,D) in bf16.  If dq_acc (fp32, contiguous (B,Sq,Hq,D)) is not NULL the block's
  * dq is ALSO added into it in fp32 -- the `reduce(op=torch.add, buffer=reduce_dq, ...)`
  * of utils/attn_bwd_dsl.py:117-122 folded into the kernel.  `workspace` must hold
- * mhip_attn_bwd_workspace_bytes(...) bytes of device memory.  dq and out have element strides of their own:
+ * mhip_attn_bwd_workspace_bytes(...) bytes of device memory: three (B, Hq, Sq) fp32 arrays, each rounded up to a
+ * multiple of 4 elements -- -delta (= -rowsum(dout * out), stored negated because the kernels start dP from it),
+ * the LSE in base 2, and delta itself, which is what flash-attn returns as softmax_d.  dq and out have element strides of their own:
  * the call site allocates block_dq with torch.empty (contiguous, utils/attn_bwd_dsl.py:83) while q, out and
  * dout are views of the step's buffers; q and dout, k and v, dk and dv share a stride triple each.
  * Head dimension: any multiple of 8 up to 128, as for the bf16 forward (for D < 128 the q / dout span of one
@@ -109,8 +115,10 @@ int mhip_attn_bwd_block(const void* dout, const void* q, const void* k, const vo
  * harnesses that forbid hipMalloc.  delta and lse2 go to an array built into the library (a file-scope
  * __device__ array of 8 MiB + 32 bytes, held by every GPU the library runs on until the process ends), so
  * the block is limited to B * Hq * Sq <= 1048576 (MHIP_ETOOLARGE beyond).  The first call on a device asks
- * the runtime for that device's address of the array (hipGetSymbolAddress, MHIP_ERUNTIME if that fails);
- * no call allocates or frees.  All calls on one GPU share the array: calls that overlap in time on one GPU
+ * the runtime for that device's address of the array (hipGetSymbolAddress, MHIP_ERUNTIME if that fails), which
+ * is a runtime query and must not happen while the stream is being captured: call mhip_init() on the device
+ * first (or make one eager call) before recording this entry point into a HIP graph.
+ * No call allocates or frees.  All calls on one GPU share the array: calls that overlap in time on one GPU
  * (different streams, different threads) race on it and must be serialised by the caller.  Arguments,
  * results and error codes are otherwise those of mhip_attn_bwd_block.
  */

@@ -26,6 +26,7 @@ _I, _L, _F, _P = c_int, c_int64, c_float, c_void_p
 _SIGNATURES = {
     "mhip_version": (c_int, []),
     "mhip_abi_version": (c_int, []),
+    "mhip_init": (c_int, []),
     "mhip_error_string": (ctypes.c_char_p, [_I]),
     "mhip_attn_fwd_block": (c_int, [_P] * 5 + [_I] * 6 + [_L] * 12 + [_F, _I, _I, _P, _P, _P, _P]),
     "mhip_attn_bwd_workspace_bytes": (c_int64, [_I] * 6),

@@ -58,7 +58,8 @@ struct BwdParams {
 // delta = rowsum(dout * out): one row of D <= 128 values per 16 lanes (8 values each); lse2 as described above
 __global__ __launch_bounds__(256) void bwd_prepare(const uint16_t* __restrict__ dout, const uint16_t* __restrict__ out,
                                                    const float* __restrict__ lse, float* __restrict__ delta,
-                                                   float* __restrict__ lse2, int B, int Sq, int Hq, int D,
+                                                   float* __restrict__ lse2, float* __restrict__ softmax_d,
+                                                   int B, int Sq, int Hq, int D,
                                                    int64_t sb, int64_t ss, int64_t sh,
                                                    int64_t o_sb, int64_t o_ss, int64_t o_sh) {
   const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
@@ -80,6 +81,7 @@ __global__ __launch_bounds__(256) void bwd_prepare(const uint16_t* __restrict__ 
   for (int m = 8; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 16);
   if (row < rows && c == 0) {      // (B, Hq, Sq) contiguous
     delta[row] = -acc;       // stored negated: the main kernels start dP^T = Y Z^T from it (C operand of the first MFMA)
+    if (softmax_d) softmax_d[row] = acc;     // the value itself, for callers that want flash-attn's softmax_d back
     const float l = lse[row];
     lse2[row] = (l == -INFINITY) ? INFINITY : l * kLog2e;
   }
@@ -566,7 +568,8 @@ using namespace mhip;
 extern "C" int64_t mhip_attn_bwd_workspace_bytes(int B, int Sq, int Sc, int Hq, int Hkv, int D) {
   (void)Sc; (void)Hkv; (void)D;
   if (B < 0 || Sq < 0 || Hq < 0) return 0;
-  return (int64_t)B * Hq * Sq * 8 + 32;     // delta and lse2, (B, Hq, Sq) fp32 each
+  // -delta, lse2 and delta, (B, Hq, Sq) fp32 each, every one starting on a 16-byte boundary
+  return ((((int64_t)B * Hq * Sq + 3) & ~int64_t(3)) * 3) * 4;
 }
 
 // Scratch of the entry point that allocates nothing: delta and lse2 of up to kScratchRows (batch, head, row)
@@ -638,7 +641,9 @@ int bwd_block(const void* dout, const void* q, const void* k, const void* v,
   p.q = static_cast<const uint16_t*>(q); p.k = static_cast<const uint16_t*>(k);
   p.v = static_cast<const uint16_t*>(v); p.dout = static_cast<const uint16_t*>(dout);
   float* delta_buf = static_cast<float*>(workspace);
-  float* lse2_buf = delta_buf + (((int64_t)B * Hq * Sq + 3) & ~int64_t(3));     // 16-byte aligned
+  const int64_t slot = ((int64_t)B * Hq * Sq + 3) & ~int64_t(3);                // 16-byte aligned
+  float* lse2_buf = delta_buf + slot;
+  float* softmax_d = own_scratch ? nullptr : lse2_buf + slot;      // the built-in scratch has no room for it
   p.lse2 = lse2_buf; p.delta = delta_buf;
   p.dq = static_cast<uint16_t*>(dq); p.dk = static_cast<uint16_t*>(dk); p.dv = static_cast<uint16_t*>(dv);
   p.dq_acc = dq_acc;
@@ -656,7 +661,7 @@ int bwd_block(const void* dout, const void* q, const void* k, const void* v,
     const int64_t rows = (int64_t)B * Hq * Sq;
     hipLaunchKernelGGL(bwd_prepare, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
                        static_cast<const uint16_t*>(dout), static_cast<const uint16_t*>(out), lse,
-                       delta_buf, lse2_buf, B, Sq, Hq, D, q_sb, q_ss, q_sh, o_sb, o_ss, o_sh);
+                       delta_buf, lse2_buf, softmax_d, B, Sq, Hq, D, q_sb, q_ss, q_sh, o_sb, o_ss, o_sh);
     // dQ: one workgroup per 128 query rows
     p.n_tiles = (Sq + kRowsPerWg - 1) / kRowsPerWg;
     p.total = B * Hq * p.n_tiles;
@@ -677,6 +682,14 @@ int bwd_block(const void* dout, const void* q, const void* k, const void* v,
   return launch_status();
 }
 }  // namespace
+
+// Resolves, for the current device, whatever the entry points otherwise look up on their first call (the address
+// of the built-in scratch): a caller that records its calls (HIP graph capture) makes this call first, outside
+// the capture.
+extern "C" int mhip_init(void) {
+  void* unused = nullptr;
+  return scratch_address(&unused);
+}
 
 extern "C" int mhip_attn_bwd_block(const void* dout, const void* q, const void* k, const void* v,
                                    const void* out, const float* lse,

@@ -195,8 +195,11 @@ def attn_bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_scale, c
     if dk_w is not dk:
         dk.copy_(dk_w)
         dv.copy_(dv_w)
-    # the workspace starts with -delta = -rowsum(dout * out), (B, Hq, Sq) fp32
-    return ws[: B * Hq * Sq * 4].view(torch.float32).view(B, Hq, Sq).neg()
+    # the workspace is (-delta | lse in base 2 | delta), (B, Hq, Sq) fp32 each in a slot rounded up to 4 elements:
+    # the last one is flash-attn's softmax_d, handed back as a view (no extra kernel, no extra allocation)
+    rows = B * Hq * Sq
+    slot = (rows + 3) & ~3
+    return ws.view(torch.float32)[2 * slot: 2 * slot + rows].view(B, Hq, Sq)
 
 
 @torch.library.custom_op("mercury_amd::_flash_attn_backward", mutates_args=("dq", "dk", "dv"),

@@ -76,3 +76,41 @@ def test_no_alloc_entry_rejects_what_does_not_fit():
                                            0.1, 0, 0, None)
     assert code == ETOOLARGE
     assert b"scratch" in lib.mhip_error_string(code)
+
+
+def test_no_alloc_entry_recorded_into_a_hip_graph():
+    """The use it is meant for: after mhip_init() (the symbol-address query, outside the capture) the call is
+    recorded into a HIP graph; every replay, with the program's own eager work and synchronisations in between
+    and the inputs rewritten in place, gives the bits of an eager call on the same inputs."""
+    import mercury_artifact_amd as M
+
+    scale = 128 ** -0.5
+    B, Sq, Sc, Hq, Hkv = 1, 256, 192, 4, 2
+    q, k, v, dout = _inputs(B, Sq, Sc, Hq, Hkv, 5)
+    out, lse = M.attn_fwd_block(q, k, v, scale)
+    dq = torch.empty_like(q)
+    dkv = torch.empty((2,) + tuple(k.shape), dtype=k.dtype, device=k.device)
+    assert N.lib().mhip_init() == 0
+
+    def call():
+        args = [N.ptr(dout), N.ptr(q), N.ptr(k), N.ptr(v), N.ptr(out), N.ptr(lse), N.ptr(dq), N.ptr(dkv[0]), N.ptr(dkv[1]),
+                None, B, Sq, Sc, Hq, Hkv, 128, q.stride(0), q.stride(1), q.stride(2),
+                k.stride(0), k.stride(1), k.stride(2), dkv[0].stride(0), dkv[0].stride(1), dkv[0].stride(2),
+                dq.stride(0), dq.stride(1), dq.stride(2), out.stride(0), out.stride(1), out.stride(2), scale, 0, 0]
+        N.check(N.lib().mhip_attn_bwd_block_noalloc(*args, N.stream_of(q)), "noalloc")
+
+    graphed = M.GraphedStep(call, warmup=0)          # recorded without an eager call before it
+    for it in range(3):
+        if it:                                        # new inputs, in place
+            g = torch.Generator().manual_seed(50 + it)
+            dout.copy_(torch.randn(dout.shape, generator=g).bfloat16())
+        torch.cuda.synchronize()
+        call()
+        torch.cuda.synchronize()
+        want = (dq.clone(), dkv.clone())
+        dq.zero_()
+        dkv.zero_()
+        torch.cuda.synchronize()
+        graphed.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(_bits(dq), _bits(want[0])) and torch.equal(_bits(dkv), _bits(want[1])), it
