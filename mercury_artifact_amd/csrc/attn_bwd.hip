@@ -265,10 +265,7 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
   // wavefront and nobody reads tile t-1 any more, whose stage then receives tile t+3.  Tiles past the end
   // are copied as zeros (and their T1 / T2 computed, unused) so that the number of copies in flight
   // stays the same.
-#ifndef MHIP_BWD_DEPTH
-#define MHIP_BWD_DEPTH 4
-#endif
-  constexpr int kDepth = MHIP_BWD_DEPTH;                   // operand reads in flight ahead of the MFMAs
+  constexpr int kDepth = 4;                                // operand reads in flight ahead of the MFMAs (2 and 8 measure the same)
   constexpr int kAcc = DQ ? 8 : 16;                        // slots of an accumulate phase
   constexpr int kP1 = 16, kP2 = 16 + kAcc, kP3 = 32 + kAcc, kSlots = 32 + 2 * kAcc;
   typedef __attribute__((address_space(3))) const bf16x8* lds_bf16x8;

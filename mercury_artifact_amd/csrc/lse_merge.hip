@@ -26,15 +26,9 @@ __device__ __forceinline__ void merge_weights(float lse, float bl, float& w, flo
   new_lse = fmaxf(lse, bl) + log1pf(e);
 }
 
-#ifndef MHIP_MERGE_NT
-#define MHIP_MERGE_NT 2      // bit 0: non-temporal accumulator loads, bit 1: non-temporal accumulator stores
-#endif
-__device__ __forceinline__ f32x4 stream_load(const f32x4* p) {
-  return (MHIP_MERGE_NT & 1) ? __builtin_nontemporal_load(p) : *p;
-}
-__device__ __forceinline__ void stream_store(f32x4 v, f32x4* p) {
-  if (MHIP_MERGE_NT & 2) __builtin_nontemporal_store(v, p); else *p = v;
-}
+// Accumulator traffic: plain loads, non-temporal stores (non-temporal loads measured slower, plain stores too).
+__device__ __forceinline__ f32x4 stream_load(const f32x4* p) { return *p; }
+__device__ __forceinline__ void stream_store(f32x4 v, f32x4* p) { __builtin_nontemporal_store(v, p); }
 
 struct MergeParams {
   const float* acc_out; const float* acc_lse;
@@ -165,10 +159,7 @@ __global__ __launch_bounds__(256) void lse_merge_generic(const MergeParams p, in
 
 template <int LPR>
 void launch_merge(const MergeParams& p, bool first, bool fin, hipStream_t st) {
-  #ifndef MHIP_MERGE_ROWS
-#define MHIP_MERGE_ROWS 2
-#endif
-  constexpr int ROWS = MHIP_MERGE_ROWS;
+  constexpr int ROWS = 2;            // rows in flight per thread (1 and 4 measured slower)
   constexpr int kRowsPerBlock = (256 / LPR) * ROWS;
   const dim3 grid((unsigned)((p.rows + kRowsPerBlock - 1) / kRowsPerBlock)), block(256);
   if (first && fin) hipLaunchKernelGGL((lse_merge_kernel<LPR, ROWS, true, true>), grid, block, 0, st, p);
@@ -183,9 +174,6 @@ void launch_merge(const MergeParams& p, bool first, bool fin, hipStream_t st) {
 // 21.9 vs 29.8 us with the fused bf16 epilogue, 21.1 vs 16.8 us for the first-call cast.  Inside a ring
 // step, where a merge follows a block forward and its operands were written just before, the plain merge
 // is faster with four values per lane (31.6 vs 33.4 us), so only the fused-epilogue merges run here.
-#ifndef MHIP_MERGE8_ROWS
-#define MHIP_MERGE8_ROWS 1
-#endif
 template <int LPR, int ROWS, bool FIRST, bool FINAL>
 __global__ __launch_bounds__(256) void lse_merge_kernel8(const MergeParams p) {
   constexpr int D = LPR * 8;
@@ -265,7 +253,7 @@ __global__ __launch_bounds__(256) void lse_merge_kernel8(const MergeParams p) {
 
 template <int LPR>
 void launch_merge8(const MergeParams& p, bool first, bool fin, hipStream_t st) {
-  constexpr int ROWS = MHIP_MERGE8_ROWS;
+  constexpr int ROWS = 1;
   constexpr int kRowsPerBlock = (256 / LPR) * ROWS;
   const dim3 grid((unsigned)((p.rows + kRowsPerBlock - 1) / kRowsPerBlock)), block(256);
   if (first && fin) hipLaunchKernelGGL((lse_merge_kernel8<LPR, ROWS, true, true>), grid, block, 0, st, p);
@@ -631,10 +619,8 @@ extern "C" int mhip_lse_merge(const float* acc_out, const float* acc_lse,
   if (dst_out) vec = vec && mult4(do_sb) && mult4(do_ss) && mult4(do_sh) && aligned16(dst_out);
   if (fin) vec = vec && (reinterpret_cast<uintptr_t>(final_out) & 7u) == 0;
   auto mult8 = [](int64_t x) { return (x & 7) == 0; };
-#ifndef MHIP_MERGE8
-#define MHIP_MERGE8 1      // 1: merges with the fused bf16 epilogue, 2: every merge but the first call, 0: none
-#endif
-  const bool vec8 = (MHIP_MERGE8 == 2 || (MHIP_MERGE8 == 1 && fin)) && vec && !first && D == 128 && mult8(bo_sb) && mult8(bo_ss) && mult8(bo_sh) && aligned16(block_out) &&
+  // eight values per lane pay for the merges with the fused bf16 epilogue only (the others measured slower in the chain)
+  const bool vec8 = fin && vec && !first && D == 128 && mult8(bo_sb) && mult8(bo_ss) && mult8(bo_sh) && aligned16(block_out) &&
                     (!fin || aligned16(final_out));
   if (vec8) {
     launch_merge8<16>(p, first, fin, st);

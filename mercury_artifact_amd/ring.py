@@ -81,12 +81,30 @@ def _fwd_params(q, k, v, softmax_scale, dropout_p, causal, window_size, alibi_sl
     return params
 
 
+_SIDE_STREAMS = {}
+
+
+def _side_stream(device) -> "torch.cuda.Stream":
+    """One extra stream per device (default priority), made on first use and kept."""
+    key = torch.device(device).index if torch.device(device).index is not None else torch.cuda.current_device()
+    if key not in _SIDE_STREAMS:
+        _SIDE_STREAMS[key] = torch.cuda.Stream(device=key)
+    return _SIDE_STREAMS[key]
+
+
 def _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes,
-                  ring: LocalRing, fused_epilogue: bool, deferred_merge: bool, ring_divide: int = 1, **extra):
+                  ring: LocalRing, fused_epilogue: bool, deferred_merge: bool, ring_divide: int = 1,
+                  two_streams: bool = False, **extra):
     """The chunk loop of the forward templates.  ``ring_divide = k > 1`` is the schedule option of the same
     name (mercury/backend/pytorch/codegen.py:299-306): an outer loop over k sub-chunks of the KV rows wraps
     the ring loop, so the step makes k * W block calls on (Sq x Sc / k) blocks and every hop moves 1/k of a
-    chunk."""
+    chunk.
+
+    ``two_streams`` (with the deferred fold only, where the block launches do not depend on each other): every
+    other block launch goes to a second stream, so that the tail of one launch (workgroups of its last round,
+    drained pipelines) overlaps the head of the next; the fold waits for both.  The side stream starts behind
+    everything queued on the current stream when the step begins; a multi-GPU ring would make it wait for the
+    hop's completion event instead."""
     blocks = []
     _out = None
     _lse = None
@@ -108,6 +126,11 @@ def _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, 
                       f"{MAX_MERGE_MANY} blocks and writes contiguous bfloat16, so this step merges block by block "
                       "(same result, one pass over the fp32 accumulator per block)", RuntimeWarning, stacklevel=3)
     done = 0
+    main = side = None
+    if two_streams and defer:
+        main = torch.cuda.current_stream(q.device)
+        side = _side_stream(q.device)
+        side.wait_stream(main)
     for part in range(ring_divide):
         rows = slice(part * sub, (part + 1) * sub)
         part_ring = ring if ring_divide == 1 else \
@@ -124,14 +147,22 @@ def _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, 
                 part_ring.commit()
             _k = _kv[0]
             _v = _kv[1]
-            outputs = _flash_attn_forward(**_fwd_params(q, _k, _v, softmax_scale, dropout_p, causal,
-                                                        window_size, alibi_slopes, **extra))
+            params = _fwd_params(q, _k, _v, softmax_scale, dropout_p, causal, window_size, alibi_slopes, **extra)
+            if side is not None and done % 2 == 1:
+                with torch.cuda.stream(side):
+                    outputs = _flash_attn_forward(**params)
+                for t in outputs[:2]:
+                    t.record_stream(main)            # allocated under the side stream, read by the fold on the main one
+            else:
+                outputs = _flash_attn_forward(**params)
             assert len(outputs) == 4
             block_out, block_lse, _, _ = outputs
             done += 1
             if defer:
                 blocks.append((block_out, block_lse))
                 if done == n_blocks:
+                    if side is not None:
+                        main.wait_stream(side)
                     merge_many([b[0] for b in blocks], [b[1] for b in blocks], o, lse)
                     return
                 continue
@@ -146,11 +177,12 @@ def _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, 
 
 def flash_attn_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False, window_size=(-1, -1),
                        alibi_slopes=None, deterministic=False, *, ring: LocalRing,
-                       fused_epilogue: bool = True, deferred_merge: bool = True, ring_divide: int = 1):
+                       fused_epilogue: bool = True, deferred_merge: bool = True, ring_divide: int = 1,
+                       two_streams: bool = False):
     """Single-ring forward step (template utils/flash_attn_dsl.py:127-180).  q (B,Sq,H,D), kv the
     rank's own (2,B,Sc,H,D), o (B,Sq,H,D) and lse (B,H,Sq) are written."""
     _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, alibi_slopes, ring,
-                  fused_epilogue, deferred_merge, ring_divide)
+                  fused_epilogue, deferred_merge, ring_divide, two_streams)
 
 
 def gqa_pack_kv(q, kv, o, lse, softmax_scale, dropout_p=0, causal=False, window_size=(-1, -1),
