@@ -74,7 +74,7 @@ def mercury_lowering() -> Lowering:
 
 def bench_program(program, namespace: Optional[dict] = None, num_iter: int = 100,
                   kwargs: Optional[dict] = None, log: bool = True, lowering: Optional[Lowering] = None,
-                  lazy_merge: bool = False) -> Tuple[float, float, int]:
+                  lazy_merge: bool = True) -> Tuple[float, float, int]:
     """Counterpart of the reference's ``bench_program`` (mercury/search/bench.py:15-86): lower ``program`` to
     source text, ``exec`` it in a namespace filled with this package's operators (``lazy_merge`` as in
     :func:`mercury_artifact_amd.namespace`), allocate one tensor per I/O buffer on this rank's device (zeros

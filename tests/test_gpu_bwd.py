@@ -199,6 +199,17 @@ def test_bwd_ring_full_size(fused):
         _check_grad(f"dk[{c}]", got[c][0][:, :, heads], rdkv[c][0])
         _check_grad(f"dv[{c}]", got[c][1][:, :, heads], rdkv[c][1])
     assert torch.equal(dkv.float(), got[rank])          # the rank's own chunk is what dkv receives
+    # every head: dQ on a window of 256 query rows (a function of those rows alone) over all chunks, and dK / dV of
+    # a 256-key window of one chunk (a sum over all query rows)
+    rows = slice(2944, 3200)
+    wdq, _ = O.ring_backward(q[:, rows].float(), [c.float() for c in kvs], order, o[:, rows].float().cpu(),
+                             lse[:, :, rows].cpu(), dout[:, rows].float(), scale)
+    _check_grad("dq, all heads", dq[:, rows], wdq)
+    c = order[3]
+    _, wdkv = O.ring_backward(q.float(), [kvs[c][:, :, 512:768].float()], [0], o.float().cpu(), lse.cpu(),
+                              dout.float(), scale)
+    _check_grad(f"dk[{c}], all heads", got[c][0][:, 512:768], wdkv[0][0])
+    _check_grad(f"dv[{c}], all heads", got[c][1][:, 512:768], wdkv[0][1])
 
 
 def test_bwd_block_head_dim_64():

@@ -50,22 +50,25 @@ def test_zigzag_causal_gqa_full_size():
         assert (o[:, rows].float() - so.float()).abs().max().item() <= 4e-3
         assert ((lse[:, :, rows] - sl).abs() / sl.abs().clamp_min(1.0)).max().item() <= 1e-5
 
-    # (2) oracle on 128-row windows: the first rows of the early block, the last rows of the late block
-    heads = [0, 17, 31]
+    # (2) oracle on 128-row windows: the first rows of the early block, the last rows of the late block; both
+    # batches, one query head of every one of the 8 K/V groups (a different member of the group each time)
+    heads = [4 * gidx + (gidx % 4) for gidx in range(Hkv)]
     kvh = [h // (Hq // Hkv) for h in heads]
-    for half, blk, first in ((0, rank, True), (1, 2 * W - 1 - rank, False)):
-        lo = half * block + (0 if first else block - 128)
-        gpos = blk * block + (0 if first else block - 128)          # global position of the window's first row
-        end = gpos + 128
-        qw = q_full_rows[1:2, lo:lo + 128][:, :, heads].float().cpu()
-        kw = k[1:2, :end][:, :, kvh].float().cpu()
-        vw = v[1:2, :end][:, :, kvh].float().cpu()
-        ro, rl = O.block_attention(qw, kw, vw, scale, causal=True)
-        go = o[1:2, lo:lo + 128][:, :, heads].float().cpu()
-        gl = lse[1:2, heads, lo:lo + 128].cpu()
-        assert (go - ro).abs().max().item() <= 2e-2
-        assert (go - ro).norm().item() / ro.norm().item() <= 1e-2
-        assert ((gl - rl).abs() / rl.abs().clamp_min(1.0)).max().item() <= 1e-3
+    assert sorted(kvh) == list(range(Hkv))
+    for bi in range(B):
+        for half, blk, first in ((0, rank, True), (1, 2 * W - 1 - rank, False)):
+            lo = half * block + (0 if first else block - 128)
+            gpos = blk * block + (0 if first else block - 128)          # global position of the window's first row
+            end = gpos + 128
+            qw = q_full_rows[bi:bi + 1, lo:lo + 128][:, :, heads].float().cpu()
+            kw = k[bi:bi + 1, :end][:, :, kvh].float().cpu()
+            vw = v[bi:bi + 1, :end][:, :, kvh].float().cpu()
+            ro, rl = O.block_attention(qw, kw, vw, scale, causal=True)
+            go = o[bi:bi + 1, lo:lo + 128][:, :, heads].float().cpu()
+            gl = lse[bi:bi + 1, heads, lo:lo + 128].cpu()
+            assert (go - ro).abs().max().item() <= 2e-2
+            assert (go - ro).norm().item() / ro.norm().item() <= 1e-2
+            assert ((gl - rl).abs() / rl.abs().clamp_min(1.0)).max().item() <= 1e-3
 
 
 def test_fp8_double_ring_full_size():
@@ -94,8 +97,8 @@ def test_fp8_double_ring_full_size():
     assert (o.float() - so.float()).abs().max().item() <= 4e-3
     assert ((lse - sl).abs() / sl.abs().clamp_min(1.0)).max().item() <= 1e-5
 
-    # (2) oracle on two heads x two 64-row windows, over all keys
-    heads = [3, 30]
+    # (2) oracle on four heads x two 64-row windows, over all keys
+    heads = [3, 12, 21, 30]
     rows = torch.cat([torch.arange(0, 64), torch.arange(Sc - 64, Sc)])
     go = o[:, rows][:, :, heads].float().cpu()
     gl = lse[:, heads][:, :, rows].cpu()

@@ -132,6 +132,38 @@ def test_fwd_block_monotone_scores(direction, fp8):
     assert ((lse - rl).abs() / rl.abs().clamp_min(1.0)).max().item() <= 1e-3
 
 
+@pytest.mark.parametrize("direction", ["rising", "falling"])
+@pytest.mark.parametrize("D", [128, 64, 40])
+@pytest.mark.parametrize("causal", [False, True])
+def test_fwd_block_monotone_scores_by_head_dim(direction, D, causal):
+    """The same ramp of about 20 binades per key tile on the 64-column instantiation (D = 64: other slot
+    arithmetic for the exponential pairs that ride in the matrix phase, the packed P overwritten right behind two
+    O^T MFMAs) and on a head dimension below 128 of the 128-column one (D = 40), with and without the causal
+    mask, so that the path that moves the reference runs together with masking.  The first 16 head-dim values
+    carry the ramp."""
+    import mercury_artifact_amd as M
+
+    B, Sq, Sc, H = 1, 320, 640, 2
+    g = torch.Generator().manual_seed(70 + D)
+    q = torch.randn(B, Sq, H, D, generator=g) * 0.25
+    k = torch.randn(B, Sc, H, D, generator=g) * 0.25
+    v = torch.randn(B, Sc, H, D, generator=g)
+    ramp = torch.arange(Sc, dtype=torch.float32) / 64.0
+    if direction == "falling":
+        ramp = ramp.flip(0)
+    scale = D ** -0.5
+    per_unit = 20.0 / (scale * 1.4426950408889634)                   # q.k increment that is 20 binades after scaling
+    q[..., :16] = 2.0
+    k[..., :16] = (ramp * per_unit / 32.0)[None, :, None, None]      # 16 columns x 2.0 x value
+    qb, kb, vb = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    ro, rl = O.block_attention(qb.float(), kb.float(), vb.float(), scale, causal=causal)
+    out, lse = M.attn_fwd_block(qb.cuda(), kb.cuda(), vb.cuda(), scale, causal=causal)
+    out, lse = out.float().cpu(), lse.cpu()
+    assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+    assert (out - ro).abs().max().item() <= 2e-2
+    assert ((lse - rl).abs() / rl.abs().clamp_min(1.0)).max().item() <= 1e-3
+
+
 def test_fwd_block_strided_views_and_guard_bands():
     """k / v as halves of one packed tensor (storage offset != 0 for v), q as a row slice of a larger
     tensor, out written into the middle of a sentinel-filled buffer."""
@@ -232,6 +264,10 @@ def test_fwd_chunks_merge_to_single_pass_full_size():
     heads = [0, 13, 31]
     ro, rl = O.block_attention(q[:, :, heads].float(), k[:, :, heads].float(), v[:, :, heads].float(), scale)
     _check(o[:, :, heads], lse[:, heads], ro, rl, "config1")
+    # every head on one window of 256 rows (rows 1792 .. 2047, across a workgroup boundary of the kernel)
+    rows = slice(1792, 2048)
+    ro, rl = O.block_attention(q[:, rows].float(), k.float(), v.float(), scale)
+    _check(o[:, rows], lse[:, :, rows], ro, rl, "config1, all heads")
 
 
 @pytest.mark.parametrize("D,causal", [(64, False), (64, True), (32, False), (96, True), (8, False), (120, True)])

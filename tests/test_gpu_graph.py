@@ -132,10 +132,29 @@ def test_search_harness_bench_program_allocates_execs_and_times(lazy, capsys):
             return super().send_recv(send_to, recv_from, tensor)
 
     extra = {"torch": torch, "dist": _Dist(rank), "WORLD": W, "SendRecv": Ring}
-    ips, seconds, mem = SH.bench_program(program, extra, num_iter=3, kwargs={"softmax_scale": D ** -0.5},
-                                         log=True, lowering=low, lazy_merge=lazy)
+    real_bench_callable = SH.bench_callable
+
+    def spy(func, call, *a, **kw):                   # the tensors the harness allocated
+        seen["call"] = call
+        return real_bench_callable(func, call, *a, **kw)
+
+    SH.bench_callable = spy
+    try:
+        ips, seconds, mem = SH.bench_program(program, extra, num_iter=3, kwargs={"softmax_scale": D ** -0.5},
+                                             log=True, lowering=low, lazy_merge=lazy)
+    finally:
+        SH.bench_callable = real_bench_callable
     assert ips > 0 and seconds > 0 and abs(ips * seconds - 3) < 1e-6 and mem == nbytes
     assert seen["kv_dtype"] == torch.bfloat16
+    # what the timed function left in the output buffers is the ring step of the oracle on the allocated inputs
+    call = seen["call"]
+    assert call["q"].dtype == torch.bfloat16 and call["lse"].dtype == torch.float32
+    chunks = [c.float().cpu() for c in other]
+    chunks[rank] = call["kv"].float().cpu()
+    import oracle as O
+    ro, rl = O.ring_forward(call["q"].float().cpu(), chunks, O.single_ring_order(rank, W), D ** -0.5)
+    assert (call["o"].float().cpu() - ro).abs().max().item() <= 2e-2
+    assert ((call["lse"].cpu() - rl).abs() / rl.abs().clamp_min(1.0)).max().item() <= 1e-3
     printed = capsys.readouterr().out
     assert "def ring_step" in printed and "iter/s" in printed and "Memory cost" in printed
 
