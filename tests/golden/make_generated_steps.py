@@ -34,8 +34,12 @@ def template_strings(path):
     return out
 
 
-def main():
-    sys.path.insert(0, REFERENCE)
+def collect(lowering=None, backward=True):
+    """The recipes as a list of dicts.  ``lowering`` (four callables: eliminate_loops, generate_code, io_buffers,
+    buffer_bytes -- the fields of mercury_artifact_amd.search_harness.Lowering) defaults to the reference's own
+    functions, called directly; ``backward=False`` leaves out the searched backward programs."""
+    if REFERENCE not in sys.path:
+        sys.path.insert(0, REFERENCE)
     import mercury.ir.loop_eliminating as le
     import mercury.ir.primitives as sp
     from mercury.backend.pytorch.codegen import generate_pytorch_code
@@ -43,7 +47,9 @@ def main():
     from mercury.ir.distributed import DeviceMesh
     from mercury.ir.init_distributed import init_distributed
     from mercury.ir.nodes import AxisDef, GridLoop
+    from mercury.ir.calculate_memory import get_buffer_size
     from mercury.ir.tile import tile_loop
+    from mercury.ir.utils import get_io_buffers
 
     templates = template_strings(os.path.join(REFERENCE, "utils", "flash_attn_dsl.py"))
     templates.update(template_strings(os.path.join(REFERENCE, "utils", "attn_bwd_dsl.py")))
@@ -66,9 +72,23 @@ def main():
         assert len(loops) == 2
         return loops
 
+    def harness_view(program):
+        """What the reference's bench_program (mercury/search/bench.py:45-60) takes from a lowered program besides
+        its text: one entry per I/O buffer (argument name, per-rank shape, dtype, written or not) and the byte count."""
+        buffers = [{"tensor": b.tensor, "shape": [int(d) for d in b.shape], "dtype": str(b.dtype).replace("torch.", ""),
+                    "write": bool(b.write)} for b in io_buffers(program)]
+        return {"io_buffers": buffers, "buffer_bytes": int(buffer_bytes(program))}
+
+    if lowering is None:
+        eliminate, generate = le.eliminate_loops, generate_pytorch_code
+        io_buffers, buffer_bytes = (lambda program: program.visit(get_io_buffers)), get_buffer_size
+    else:
+        eliminate, generate = lowering.eliminate_loops, lowering.generate_code
+        io_buffers, buffer_bytes = lowering.io_buffers, lowering.buffer_bytes
+
     def finish(program):
-        le.eliminate_loops(program)
-        return program.name, generate_pytorch_code(program)
+        eliminate(program)
+        return program.name, generate(program), harness_view(program)
 
     fwd = dict(BATCH=B, SEQ_LEN=S, HEADS=H, HEAD_DIM=D)
     red = dict(fwd, RED_DIM=D + 1)
@@ -76,10 +96,10 @@ def main():
 
     def recipe(name, source, mesh_shape, q_dims, kv_dims, heads_q=H, heads_kv=H):
         def deco(fn):
-            program_name, code = fn()
+            program_name, code, view = fn()
             recipes.append({"name": name, "source": source, "mesh": list(mesh_shape), "function": program_name,
                             "q_dims": list(q_dims), "kv_dims": list(kv_dims), "B": B, "S": S, "Hq": heads_q,
-                            "Hkv": heads_kv, "D": D, "code": code})
+                            "Hkv": heads_kv, "D": D, "code": code, **view})
             return fn
         return deco
 
@@ -199,15 +219,17 @@ def main():
 
     # ---- backward: the schedules the reference's search finds on a 1-D mesh (tests/test_attn_bwd.py:53-130 runs
     # every searched program); one of each kind, with all heads on every rank -----------------------------------------
+    if not backward:
+        return recipes
     import re
 
     from mercury.search.search import search
 
     program = parse("attn_backward_template", **fwd)
-    found = set()
+    found = {}
     for candidate in search(program, DeviceMesh(list(range(4)), (4,)), ["S_q", "S_kv"]):
-        le.eliminate_loops(candidate)
-        found.add(generate_pytorch_code(candidate))
+        eliminate(candidate)
+        found.setdefault(generate(candidate), harness_view(candidate))
     # The search also tiles the two sequence loops into sub-chunks.  Taken here: per kind the untiled program, and
     # the one whose K/V loop alone is tiled.  Left out: programs with a tiled QUERY loop around a travelling dK/dV
     # buffer -- their text restarts the buffer at every query tile (`reduce_dkv[...] = block_dkv...` at ring step
@@ -237,8 +259,14 @@ def main():
     for kind, (code, nq, nkv) in sorted(kinds.items()):
         recipes.append({"name": kind, "source": "tests/test_attn_bwd.py:53-130 (mercury.search.search on a 4-rank mesh)",
                         "mesh": [4], "function": program.name, "q_dims": [0] if nq == 4 else [],
-                        "kv_dims": [0] if nkv == 4 else [], "B": B, "S": S, "Hq": H, "Hkv": H, "D": D, "code": code})
+                        "kv_dims": [0] if nkv == 4 else [], "B": B, "S": S, "Hq": H, "Hkv": H, "D": D, "code": code,
+                        **found[code]})
 
+    return recipes
+
+
+def main():
+    recipes = collect()
     out = os.path.join(HERE, "generated_steps.json")
     with open(out, "w") as fh:
         json.dump({"made_by": "tests/golden/make_generated_steps.py", "recipes": recipes}, fh, indent=1)

@@ -148,3 +148,70 @@ def test_generated_backward_step_of_every_rank_matches_the_oracle(recipe):
         assert rel(dq, rdq.chunk(qn, dim=1)[qi]) <= 1e-2, rank
         assert rel(dkv[0], rdk.chunk(kn, dim=1)[ki]) <= 1e-2, rank
         assert rel(dkv[1], rdv.chunk(kn, dim=1)[ki]) <= 1e-2, rank
+
+
+@pytest.mark.parametrize("name", ["single_ring_divide_2", "backward_kv_ring"])
+def test_bench_program_allocates_from_the_reference_buffer_table_and_times_every_rank(name):
+    """The search's timing harness (mercury/search/bench.py:15-86) on the reference's own lowering results: the text
+    and the I/O buffer table of the fixture stand in for the four lowering calls, every rank of the mesh runs
+    ``bench_program`` (zeros for written buffers, N(0,1) for the others, warm-up and timed calls), and what the timed
+    function left in each rank's output buffers is the oracle's result on the tensors the harness allocated."""
+    import threading
+    import types
+
+    import mercury_artifact_amd as M
+    from mercury_artifact_amd import search_harness as SH
+
+    recipe = next(r for r in RECIPES if r["name"] == name)
+    W, D = recipe["mesh"][0], recipe["D"]
+    scale = D ** -0.5
+    mesh = M.LocalMesh(tuple(recipe["mesh"]))
+    buffers = [types.SimpleNamespace(tensor=b["tensor"], shape=tuple(b["shape"]), dtype=getattr(torch, b["dtype"]),
+                                     write=b["write"]) for b in recipe["io_buffers"]]
+    low = SH.Lowering(eliminate_loops=lambda prog: None, generate_code=lambda prog: _function_text(recipe["code"]),
+                      io_buffers=lambda prog: buffers, buffer_bytes=lambda prog: recipe["buffer_bytes"])
+    os.environ.setdefault("LOCAL_RANK", "0")
+    calls, timings = {}, {}
+    real_bench_callable = SH.bench_callable
+
+    def spy(func, call, *a, **kw):                   # the tensors the harness allocated, per rank thread
+        calls[threading.get_ident()] = call
+        return real_bench_callable(func, call, *a, **kw)
+
+    def rank_fn(rank):
+        extra = {"torch": torch, "os": os, "dist": mesh.dist, "SendRecv": mesh.SendRecv}
+        timings[rank] = SH.bench_program(types.SimpleNamespace(name=recipe["function"]), extra, num_iter=2,
+                                         kwargs={"softmax_scale": scale}, log=False, lowering=low)
+        calls[rank] = calls.pop(threading.get_ident())
+
+    SH.bench_callable = spy
+    try:
+        mesh.run(rank_fn)
+    finally:
+        SH.bench_callable = real_bench_callable
+    torch.cuda.synchronize()
+    assert sorted(calls) == list(range(W))
+    for rank in range(W):
+        ips, seconds, mem = timings[rank]
+        assert ips > 0 and seconds > 0 and mem == recipe["buffer_bytes"]
+        for b in buffers:
+            t = calls[rank][b.tensor]
+            assert tuple(t.shape) == b.shape and t.dtype == b.dtype and t.is_cuda
+
+    def whole(tensor, dim):                          # the ranks' shards as one sequence
+        return torch.cat([calls[r][tensor].float().cpu() for r in range(W)], dim=dim)
+
+    q, kv = whole("q", 1), whole("kv", 2)
+    if name.startswith("backward"):
+        rdq, rdk, rdv = O.block_backward(whole("dout", 1), q, kv[0], kv[1], whole("o", 1), whole("lse", 2), scale)
+        for rank in range(W):
+            dq, dkv = calls[rank]["dq"].float().cpu(), calls[rank]["dkv"].float().cpu()
+            for got, want in ((dq, rdq.chunk(W, dim=1)[rank]), (dkv[0], rdk.chunk(W, dim=1)[rank]),
+                              (dkv[1], rdv.chunk(W, dim=1)[rank])):
+                assert (got - want).norm().item() / want.norm().item() <= 1e-2, rank
+    else:
+        ro, rl = O.block_attention(q, kv[0], kv[1], scale)
+        for rank in range(W):
+            want_o, want_l = ro.chunk(W, dim=1)[rank], rl.chunk(W, dim=2)[rank]
+            assert (calls[rank]["o"].float().cpu() - want_o).abs().max().item() <= 2e-2, rank
+            assert ((calls[rank]["lse"].cpu() - want_l).abs() / want_l.abs().clamp_min(1.0)).max().item() <= 1e-3, rank
