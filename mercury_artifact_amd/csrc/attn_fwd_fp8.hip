@@ -14,9 +14,10 @@
 //     lane's 16 accumulator registers hold 16 CONSECUTIVE keys (16 hf + i): the transposing reads, which
 //     deliver 8 consecutive keys, then produce V^T in exactly the key order of the P registers;
 //   * the descales fold into the softmax scale (q, k) and the final normalisation (v);
-//   * P is multiplied by 2^7 before it is rounded to e4m3 (and the result divided by 2^7), so that small
-//     probabilities keep their relative precision; the reference score only lags the running maximum by
-//     at most one binade, which keeps 2^7 P below the e4m3 maximum of 448.
+//   * P is multiplied by 2^4 before it is rounded to e4m3 (and the result divided by 2^4), so that small
+//     probabilities keep their relative precision; the reference score of a row is its first tile's maximum
+//     and moves only when the sum of a group of 16 values of 2^4 P reaches the e4m3 maximum of 448 (the sums
+//     are watched, not the maxima: the common path has no maximum, no cross-lane exchange, no rescale of O).
 #include "mhip_common.hpp"
 
 namespace mhip {
@@ -33,8 +34,8 @@ constexpr int kTileBytes = kBN * kD;  // 16384: one K or V tile in LDS, 128 rows
 constexpr int kStages = 4;
 constexpr int kVBase = kStages * kTileBytes;
 constexpr int kOStride = kD + 8;
-constexpr float kPShift = 7.f;        // P is stored as 2^7 P in e4m3
-constexpr float kRescaleSlack = 1.f;
+constexpr float kPShift = 4.f;        // P is stored as 2^4 P in e4m3
+constexpr float kTrigger = 448.f;     // the e4m3 maximum: a group of 16 exponentials has to sum to less
 constexpr int kNoColumn = 0x7fff0000;  // vector offset that is out of every descriptor's range (spans stay below 2^30
                                        // when it is used, and so does the scalar tile offset added to it)
 
@@ -185,9 +186,65 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 16; ++j) o_acc[i][j] = 0.f;
-  float m_ref = -INFINITY, l_run = 0.f;      // l_run sums 2^7 P (this lane's half of the keys)
+  // m_ref: the raw score the exponentials of this lane's Q row are taken relative to.  It is set to the first
+  // tile's row maximum and moves only when a later tile would overflow e4m3: what is watched is the sum of each
+  // group of 16 exponentials (one compare per tile), not the maxima.  A group sum below 448 means every 2^4 P in
+  // it is below the e4m3 maximum; P = 1 for all 16 gives 256.  When a sum reaches 448 the reference moves up to
+  // the row maximum seen so far (O and the running sum are rescaled) and the tile's exponentials are redone, after
+  // which every 2^4 P is at most 16.
+  float m_ref = 0.f, msc = -kPShift, l_run = 0.f;      // l_run sums 2^4 P (this lane's half of the keys)
+  float rs_sum = 0.f;
   i32x8 pf[2] = {};          // P^T operands; pf[ks2]: dwords 0-3 = keys of block 2 ks2, dwords 4-7 = block 2 ks2 + 1
   const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  f32x16 s[4];               // S^T tile: 128 keys x 32 q rows per wave
+  auto set_reference = [&](bool first) {
+    float mx = s[0][0];
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) mx = fmaxf(mx, s[mb][j]);
+    mx = pair_max(mx);
+    const bool move = first ? (mx != -INFINITY) : (mx > m_ref);      // false for NaN
+    if (!first) {
+      const float alpha = move ? fast_exp2((m_ref - mx) * scale_log2) : 1.f;
+      l_run *= alpha;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) o_acc[db][j] *= alpha;
+    }
+    m_ref = move ? mx : m_ref;
+    msc = m_ref * scale_log2 - kPShift;            // exponent of 2^4 P
+  };
+  // 2^4 P of the tile into the P^T operands; returns whether one of the four group sums reached the trigger (or is
+  // inf / NaN) and leaves their total in rs_sum.  s stays intact, so that the pass can be repeated against a new
+  // reference.
+  auto exponentials = [&]() -> bool {
+    bool big = false;
+    rs_sum = 0.f;
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) {
+      float e[16];
+      float r = 0.f;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        e[j] = fast_exp2(__builtin_fmaf(s[mb][j], scale_log2, -msc));
+        r += e[j];
+      }
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        // the first conversion writes the low half and the second the high half of the operand register, so
+        // what it held before (the P of the previous tile) needs no clearing
+        int packed = pf[mb >> 1][(mb & 1) * 4 + w];
+        packed = __builtin_amdgcn_cvt_pk_fp8_f32(e[4 * w], e[4 * w + 1], packed, false);
+        packed = __builtin_amdgcn_cvt_pk_fp8_f32(e[4 * w + 2], e[4 * w + 3], packed, true);
+        pf[mb >> 1][(mb & 1) * 4 + w] = packed;
+      }
+      big = big || !(r < kTrigger);
+      rs_sum += r;
+    }
+    return big;
+  };
 
   // Tile t lives in stage t % 4 of the K and the V ring.  An iteration starts by waiting for this
   // wavefront's copies of tile t (those of tiles t+1 and t+2 stay in flight) and a barrier: after it tile t
@@ -221,8 +278,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
     const unsigned char* ks_ = smem + (t & 3) * kTileBytes;
     const unsigned char* vs_ = smem + kVBase + (t & 3) * kTileBytes;
 
-    // ---- S^T tile: 128 keys x 32 q rows per wave ------------------------------------------------------
-    f32x16 s[4];
+    // ---- S^T tile ---------------------------------------------------------------------------------------
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
@@ -247,45 +303,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
         }
     }
 
-    // ---- online softmax ------------------------------------------------------------------------------------
-    float mx = s[0][0];
-#pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-      for (int j = 0; j < 16; ++j) mx = fmaxf(mx, s[mb][j]);
-    mx = pair_max(mx);
-    const bool grow = (mx - m_ref) * scale_log2 > kRescaleSlack;
-    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-      const float m_new = grow ? mx : m_ref;
-      const float alpha = (m_new == -INFINITY) ? 1.f : fast_exp2((m_ref - m_new) * scale_log2);
-      m_ref = m_new;
-      l_run *= alpha;
-#pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) o_acc[db][j] *= alpha;
+    // ---- softmax against a reference that moves only when it has to -----------------------------------------
+    if (t == 0) set_reference(true);
+    if (__builtin_amdgcn_ballot_w64(exponentials()) != 0) {
+      set_reference(false);
+      exponentials();
     }
-    const float msc = (m_ref == -INFINITY) ? 0.f : m_ref * scale_log2 - kPShift;   // exponent of 2^7 P
-    float rs = 0.f;
-#pragma unroll
-    for (int mb = 0; mb < 4; ++mb) {
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const float e = fast_exp2(__builtin_fmaf(s[mb][j], scale_log2, -msc));
-        rs += e;
-        s[mb][j] = e;
-      }
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        // the first conversion writes the low half and the second the high half of the operand register, so
-        // what it held before (the P of the previous tile) needs no clearing
-        int packed = pf[mb >> 1][(mb & 1) * 4 + w];
-        packed = __builtin_amdgcn_cvt_pk_fp8_f32(s[mb][4 * w], s[mb][4 * w + 1], packed, false);
-        packed = __builtin_amdgcn_cvt_pk_fp8_f32(s[mb][4 * w + 2], s[mb][4 * w + 3], packed, true);
-        pf[mb >> 1][(mb & 1) * 4 + w] = packed;
-      }
-    }
-    l_run += rs;
+    l_run += rs_sum;
 
     // ---- O^T += V^T P^T -----------------------------------------------------------------------------------
 #pragma unroll
@@ -301,7 +325,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_fwd_fp8_d128(const Fp8Par
 
   // ---- epilogue ---------------------------------------------------------------------------------------------
   const float l_tot = pair_sum(l_run);
-  const float inv = l_tot > 0.f ? out_mul / l_tot : 0.f;           // the two factors 2^7 cancel
+  const float inv = l_tot > 0.f ? out_mul / l_tot : 0.f;           // the two factors 2^4 cancel
   if (hf == 0 && my_q < p.Sq) {
     const float lse = l_tot > 0.f ? m_ref * scale_eff + (fast_log2(l_tot) - kPShift) * kLn2 : -INFINITY;
     p.lse[((int64_t)b * p.Hq + hq) * p.Sq + my_q] = lse;

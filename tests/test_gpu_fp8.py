@@ -70,6 +70,41 @@ def test_fp8_block_matches_oracle(B, Sq, Sc, Hq, Hkv, causal):
     _check(out, lse, ref_a, ref_b, "fp8 block", p_bound, check_b=Sc >= 1000)
 
 
+@pytest.mark.parametrize("direction", ["rising", "falling"])
+@pytest.mark.parametrize("binades_per_tile", [0.75, 6.0])
+@pytest.mark.parametrize("causal", [False, True])
+def test_fp8_block_monotone_scores(direction, binades_per_tile, causal):
+    """Scores that climb (or fall) steadily from one 128-key tile to the next.  The kernel keeps the first tile's row
+    maximum as the reference of its exponentials and watches the sums of groups of 16 values of 2^4 P instead of the
+    maxima: a slow climb (0.75 binades per tile) makes a group sum reach the e4m3 maximum while every single value
+    is still below it, a steep one (6 binades) overflows single values; falling scores leave the reference where it
+    is and send the later tiles towards the small end of e4m3."""
+    import mercury_artifact_amd as M
+
+    B, Sq, Sc, H, D = 1, 320, 1024, 2, 128
+    print(f"fp8 monotone {direction} {binades_per_tile} causal={causal}", flush=True)
+    g = torch.Generator().manual_seed(91)
+    q = torch.randn(B, Sq, H, D, generator=g) * 0.25
+    k = torch.randn(B, Sc, H, D, generator=g) * 0.25
+    v = torch.randn(B, Sc, H, D, generator=g)
+    ramp = torch.arange(Sc, dtype=torch.float32) / 128.0
+    if direction == "falling":
+        ramp = ramp.flip(0)
+    scale = D ** -0.5
+    per_unit = binades_per_tile / (scale * 1.4426950408889634)      # q.k increment that is that many binades after scaling
+    q[..., :16] = 2.0
+    k[..., :16] = (ramp * per_unit / 32.0)[None, :, None, None]     # 16 columns x 2.0 x value
+    (qq, sq), (kq, sk), (vq, sv) = O.quantize_e4m3(q), O.quantize_e4m3(k), O.quantize_e4m3(v)
+    deq = (O.dequantize(qq, sq), O.dequantize(kq, sk), O.dequantize(vq, sv))
+    ref_a = O.block_attention(*deq, scale, causal=causal)
+    out, lse = M.attn_fwd_block(qq.cuda(), kq.cuda(), vq.cuda(), scale, causal=causal, q_descale=sq.cuda(),
+                                k_descale=sk.cuda(), v_descale=sv.cuda())
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    p_bound = O.e4m3_p_rounding_bound(*deq, scale, causal=causal)
+    _check(out, lse, ref_a, ref_a, f"fp8 {direction} {binades_per_tile}", p_bound, check_b=False)
+
+
 @pytest.mark.parametrize("D,causal", [(64, False), (48, True), (16, False), (112, True)])
 def test_fp8_block_smaller_head_dims(D, causal):
     """Head dimensions below 128 (multiples of 16) through the e4m3 kernel: q, k, v and out are COLUMN slices of
