@@ -270,9 +270,21 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
   constexpr int kP1 = 16, kP2 = 16 + kAcc, kP3 = 32 + kAcc, kSlots = 32 + 2 * kAcc;
   typedef __attribute__((address_space(3))) const bf16x8* lds_bf16x8;
   typedef __attribute__((address_space(3))) const f32x4* lds_f32x4;
+  // LDS addresses of the operand reads.  rm_a / tr_a hold, per lane, the addresses inside ONE tile's stage and are
+  // moved on to the next stage in place, each at a point of the slot sequence where no read of its kind is due
+  // (rm_a in slots 12-15: the reads of the current tile's T1 / T2 operands are all issued by slot 11 and those of
+  // the next tile start at slot kP2 - kDepth; tr_a in the last kDepth slots, after the last transposed read).
+  // ld_cur / ld_next address lse2 / -delta of the current and the next tile.  Everything else about an address
+  // is an immediate offset of the LDS instruction.
+  int rm_a[8], tr_a[4][2];
+#pragma unroll
+  for (int kk = 0; kk < 8; ++kk) rm_a[kk] = rm_rd[kk] + (int)lds_base;
+#pragma unroll
+  for (int db = 0; db < 4; ++db) { tr_a[db][0] = tr_rd[db][0] + (int)lds_base; tr_a[db][1] = tr_rd[db][1] + (int)lds_base; }
+  int ld_cur = (int)lds_base + hf * 16, ld_next = ld_cur + kStageBytes;
   // slot i (0..15) of the T1 / T2 sequence of one half: k-step i / 2, X (T1) on even and Y (T2) on odd slots
-  auto read_rm = [&](const int (&rm)[8], int mb, int i) -> bf16x8 {
-    return *(lds_bf16x8)(uintptr_t)(uint32_t)(rm[i >> 1] + mb * 8192 + ((i & 1) ? kOffY : 0));
+  auto read_rm = [&](int mb, int i) -> bf16x8 {
+    return *(lds_bf16x8)(uintptr_t)(uint32_t)(rm_a[i >> 1] + mb * 8192 + ((i & 1) ? kOffY : 0));
   };
   // T2 starts from -delta of the half's streamed rows (dQ pass: of this lane's stationary row), so that what
   // the vector unit receives is dP - delta already
@@ -282,27 +294,18 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     if (i & 1) n2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, yf[kk], kk == 0 ? nd : n2, 0, 0, 0);
     else n1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, xf[kk], kk == 0 ? zero : n1, 0, 0, 0);
   };
-  // LDS byte addresses of the operand reads for the tile in `stage`
-  auto tile_addrs = [&](int stage, int (&rm)[8], int (&tr)[4][2]) {
-    const int base = (int)lds_base + stage * kStageBytes;
-#pragma unroll
-    for (int kk = 0; kk < 8; ++kk) rm[kk] = rm_rd[kk] + base;
-#pragma unroll
-    for (int db = 0; db < 4; ++db) { tr[db][0] = tr_rd[db][0] + base; tr[db][1] = tr_rd[db][1] + base; }
-  };
   // slot i of an accumulate phase of half mb: head-dim block and k-step, X^T (dS) / Y^T (P) alternating for dK, dV
-  auto read_acc = [&](const int (&tr)[4][2], int mb, int i) -> bf16x8 {
+  auto read_acc = [&](int mb, int i) -> bf16x8 {
     const int m = DQ ? i : (i >> 1);
     const int off = mb * 8192 + (m >> 2) * 4096 + ((!DQ && (i & 1)) ? kOffY : 0);
-    const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4)(uintptr_t)(uint32_t)(tr[m & 3][0] + off));
-    const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4)(uintptr_t)(uint32_t)(tr[m & 3][1] + off));
+    const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4)(uintptr_t)(uint32_t)(tr_a[m & 3][0] + off));
+    const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4)(uintptr_t)(uint32_t)(tr_a[m & 3][1] + off));
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   };
 
   bf16x8 pfrag[2], dsfrag[2];     // P and dS of the half being accumulated as B operands (two k-steps)
   bf16x8 ring[kDepth];
   f32x16 ta1, ta2, tb1, tb2;      // T1 / T2 of the two halves in flight: (t, first half), (t, second half)
-  int rm_c[8], tr_c[4][2], rm_n[8], tr_n[4][2];
   f32x4 lv[5];                    // lse2 of 4 streamed rows per entry (dK / dV pass), read one group ahead
 
   // Hidden elements (rows past the end of the streamed tensor, the causal mask) get a score of -inf,
@@ -320,16 +323,14 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
       }
     }
   };
-  // lse2 / delta of rows 8 g + 4 hf .. + 3 of half mb of the tile in `stage`
-  auto read_ld = [&](int stage, int mb, int g, f32x4& l) {
-    const int addr = (int)lds_base + stage * kStageBytes + kOffLse + (mb * 32 + g * 8 + hf * 4) * 4;
-    l = *(lds_f32x4)(uintptr_t)(uint32_t)addr;
+  // lse2 of rows 8 g + 4 hf .. + 3 of half mb of the current (next: of the following) tile
+  auto read_ld = [&](bool next, int mb, int g, f32x4& l) {
+    l = *(lds_f32x4)(uintptr_t)(uint32_t)((next ? ld_next : ld_cur) + kOffLse + (mb * 32 + g * 8) * 4);
   };
-  // -delta of rows 8 g + 4 hf .. + 3 (g = 0..3) of half mb of the tile in `stage`, in the order of the
+  // -delta of rows 8 g + 4 hf .. + 3 (g = 0..3) of half mb of the current / following tile, in the order of the
   // accumulator registers of T2 (dK / dV pass), one group per call
-  auto read_nd = [&](int stage, int mb, int g) {
-    const int addr = (int)lds_base + stage * kStageBytes + kOffDelta + (mb * 32 + g * 8 + hf * 4) * 4;
-    const f32x4 d = *(lds_f32x4)(uintptr_t)(uint32_t)addr;
+  auto read_nd = [&](bool next, int mb, int g) {
+    const f32x4 d = *(lds_f32x4)(uintptr_t)(uint32_t)((next ? ld_next : ld_cur) + kOffDelta + (mb * 32 + g * 8) * 4);
 #pragma unroll
     for (int e = 0; e < 4; ++e) nd[4 * g + e] = d[e];
   };
@@ -348,7 +349,7 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     return e < 8 ? (e * 7) / 4 : 5 + e;                  // 0,1,3,5,7,8,10,12 | 13..20: packed at slots 15 and 23 (acc 16-23, 24-31)
   };
   float earg[16];
-  auto vector_slot = [&](int s, f32x16& c1, f32x16& c2, int stage, int mb) {
+  auto vector_slot = [&](int s, f32x16& c1, f32x16& c2, int mb) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int f = first_slot(e);
@@ -356,7 +357,7 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
         const float l = DQ ? lse2_lane : lv[e >> 2][e & 3];
         earg[e] = __builtin_fmaf(c1[e], p.scale_log2, -l);
         // lse2 of the next four rows, one group ahead
-        if (!DQ && (e & 3) == 0 && e < 12) read_ld(stage, mb, (e >> 2) + 1, lv[(e >> 2) + 1]);
+        if (!DQ && (e & 3) == 0 && e < 12) read_ld(false, mb, (e >> 2) + 1, lv[(e >> 2) + 1]);
       }
       if (s == f + 1) c1[e] = fast_exp2(earg[e]);
       if (s == f + 2) c2[e] = c1[e] * c2[e];
@@ -381,14 +382,16 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     if (DQ || !(i & 1)) acc1[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, dsfrag[j2], acc1[db], 0, 0, 0);
     else acc2[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pfrag[j2], acc2[db], 0, 0, 0);
   };
-  // LDS operand of slot s of the current tile's sequence; s >= kSlots continues into the next tile's P0
+  // LDS operand of slot s of the current tile's sequence; s >= kSlots continues into the next tile's P0.  The
+  // T1 / T2 operands of slots kP2 .. kP3 - 1 and from kSlots on belong to the next tile: rm_a has moved on by then.
   auto read_slot = [&](int s) -> bf16x8 {
-    if (s >= kSlots) return read_rm(rm_n, 1, s - kSlots);
-    if (s < kP1) return read_rm(rm_c, 1, s);
-    if (s < kP2) return read_acc(tr_c, 0, s - kP1);
-    if (s < kP3) return read_rm(rm_n, 0, s - kP2);
-    return read_acc(tr_c, 1, s - kP3);
+    if (s >= kSlots) return read_rm(1, s - kSlots);
+    if (s < kP1) return read_rm(1, s);
+    if (s < kP2) return read_acc(0, s - kP1);
+    if (s < kP3) return read_rm(0, s - kP2);
+    return read_acc(1, s - kP3);
   };
+  static_assert(kP2 - kDepth >= 16 && kP1 - kDepth <= 12, "rm_a moves in slots 12-15");
 
   if (ntiles > 0) {
     copy_tile(0, 0);
@@ -429,55 +432,57 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     else asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
     static_assert(kCopiesPerTile == (DQ ? 8 : 9), "the vmcnt immediates are one and two tiles of copies");
     __builtin_amdgcn_s_barrier();
-    tile_addrs(0, rm_c, tr_c);
     if (DQ) {
 #pragma unroll
       for (int j = 0; j < 16; ++j) nd[j] = delta_lane;
     } else {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) read_nd(0, 0, g);
+      for (int g = 0; g < 4; ++g) read_nd(false, 0, g);
     }
     // T1 / T2 of the first half of tile 0, nothing to interleave with
 #pragma unroll
-    for (int i = 0; i < kDepth; ++i) ring[i] = read_rm(rm_c, 0, i);
+    for (int i = 0; i < kDepth; ++i) ring[i] = read_rm(0, i);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       t_mfma(i, ring[i % kDepth], ta1, ta2);
-      if (i + kDepth < 16) ring[i % kDepth] = read_rm(rm_c, 0, i + kDepth);
+      if (i + kDepth < 16) ring[i % kDepth] = read_rm(0, i + kDepth);
     }
 #pragma unroll
-    for (int i = 0; i < kDepth; ++i) ring[i] = read_rm(rm_c, 1, i);      // slots 0 .. 3 of tile 0
+    for (int i = 0; i < kDepth; ++i) ring[i] = read_rm(1, i);            // slots 0 .. 3 of tile 0
     if (!DQ) {
-      read_ld(0, 0, 0, lv[0]);
+      read_ld(false, 0, 0, lv[0]);
 #pragma unroll
-      for (int g = 0; g < 4; ++g) read_nd(0, 1, g);            // for T2 of the second half, first thing in the loop
+      for (int g = 0; g < 4; ++g) read_nd(false, 1, g);        // for T2 of the second half, first thing in the loop
     }
   }
   for (int t = 0; t < ntiles; ++t) {
     const int c0 = tile_row0(t);
-    const int stage = t & 3;
     if (DQ) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     copy_setup(t + 3);
-    const int next_base = (int)lds_base + ((t + 1) & 3) * kStageBytes;
+    // byte distance from this tile's stage to the next tile's, and from that one to the one after
+    const int step1 = ((t + 1) & 3) == 0 ? -3 * kStageBytes : kStageBytes;
+    const int step2 = ((t + 2) & 3) == 0 ? -3 * kStageBytes : kStageBytes;
     static_assert(kSlots % kDepth == 0 && 16 % kDepth == 0, "the ring position is the slot number modulo its depth");
     mask_half(ta1, c0);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {                       // P0, carrying the copies of tile t+3
       t_mfma(i, ring[i % kDepth], tb1, tb2);
-      vector_slot(i, ta1, ta2, stage, 0);
+      vector_slot(i, ta1, ta2, 0);
       if (i < kCopiesPerTile) copy_piece(i, (t + 3) & 3);
-      if (i >= 8) rm_n[i - 8] = rm_rd[i - 8] + next_base;          // needed from P2 on (after slot kP2 - kDepth)
       ring[i % kDepth] = read_slot(i + kDepth);
+      if (i >= 12) { rm_a[2 * (i - 12)] += step1; rm_a[2 * (i - 12) + 1] += step1; }      // on to the next tile
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int i = 0; i < kAcc; ++i) {                     // P1
-      if (i < kVecTail) vector_slot(16 + i, ta1, ta2, stage, 0);
+      if (i < kVecTail) vector_slot(16 + i, ta1, ta2, 0);
       acc_mfma(i, ring[(kP1 + i) % kDepth]);
-      if (!DQ && i == kAcc - 2) read_ld(stage, 1, 0, lv[0]);
-      if (!DQ && i >= 2 && i < 6) read_nd((t + 1) & 3, 0, i - 2);      // T2 of (t+1, first half) starts in P2
+      if (!DQ && i == kAcc - 2) read_ld(false, 1, 0, lv[0]);
+      // -delta for T2 of (t+1, first half), which starts in P2: read once the vector work on this half's dP is
+      // through (slot 7), so that the values can land in the registers T2 accumulates in
+      if (!DQ && i >= 8 && i < 12) read_nd(true, 0, i - 8);
       ring[(kP1 + i) % kDepth] = read_slot(kP1 + i + kDepth);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -485,24 +490,25 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) {                       // P2
       t_mfma(i, ring[(kP2 + i) % kDepth], ta1, ta2);
-      vector_slot(i, tb1, tb2, stage, 1);
-      if (i < 8) { const int db = i >> 1, h = i & 1; tr_n[db][h] = tr_rd[db][h] + next_base; }   // for the next tile
+      vector_slot(i, tb1, tb2, 1);
       ring[(kP2 + i) % kDepth] = read_slot(kP2 + i + kDepth);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int i = 0; i < kAcc; ++i) {                     // P3
-      if (i < kVecTail) vector_slot(16 + i, tb1, tb2, stage, 1);
+      if (i < kVecTail) vector_slot(16 + i, tb1, tb2, 1);
       acc_mfma(i, ring[(kP3 + i) % kDepth]);
-      if (!DQ && i == kAcc - 2) read_ld((t + 1) & 3, 0, 0, lv[0]);
-      if (!DQ && i >= 2 && i < 6) read_nd((t + 1) & 3, 1, i - 2);      // T2 of (t+1, second half): P0 of the next tile
+      if (!DQ && i == kAcc - 2) read_ld(true, 0, 0, lv[0]);
+      if (!DQ && i >= 8 && i < 12) read_nd(true, 1, i - 8);            // T2 of (t+1, second half): P0 of the next tile
       ring[(kP3 + i) % kDepth] = read_slot(kP3 + i + kDepth);
+      if (i >= kAcc - kDepth) {                          // the last transposed read of this tile has been issued
+        const int db = i - (kAcc - kDepth);
+        tr_a[db][0] += step1; tr_a[db][1] += step1;
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
-#pragma unroll
-    for (int kk = 0; kk < 8; ++kk) rm_c[kk] = rm_n[kk];
-#pragma unroll
-    for (int db = 0; db < 4; ++db) { tr_c[db][0] = tr_n[db][0]; tr_c[db][1] = tr_n[db][1]; }
+    ld_cur = ld_next;
+    ld_next += step2;
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the zero-filled copies of tiles past the end
 
