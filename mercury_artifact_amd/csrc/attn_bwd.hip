@@ -9,8 +9,9 @@
 //                key) turned into +inf so that P = exp2(s - lse2) = 0 there       (bandwidth bound)
 //   bwd_main<DQ=false>  one workgroup per 128 keys of one KV head: K and V rows stay in registers,
 //                Q / dout tiles of the (grouped) query heads stream through LDS; accumulates dK, dV
-//   bwd_main<DQ=true>   one workgroup per 128 query rows of one head: Q and dout rows stay in registers,
-//                K / V tiles stream through LDS; accumulates dQ
+//   bwd_main<DQ=true>   one workgroup per 256 query rows of one head (eight wavefronts, two per SIMD: this pass
+//                has half the accumulators of the other and fits 256 registers): Q and dout rows stay in
+//                registers, K / V tiles stream through LDS; accumulates dQ
 // Both instances share one body.  "Stationary" rows (32 per wavefront) sit in the lane index of every
 // MFMA accumulator, "streamed" rows in its registers, exactly as in the forward kernel:
 //     T1[c][r] = X_str[c] . X_st[r]      (scores)          T2[c][r] = Y_str[c] . Y_st[r]      (dP)
@@ -30,7 +31,8 @@ namespace {
 
 constexpr int kD = 128;
 constexpr int kTile = 64;             // streamed rows per main-loop tile
-constexpr int kRowsPerWg = 128;       // stationary rows per workgroup (4 wavefronts x 32)
+constexpr int kRowsKv = 128;          // stationary key rows per workgroup of the dK / dV pass (4 wavefronts x 32)
+constexpr int kRowsQ = 256;           // stationary query rows per workgroup of the dQ pass (8 wavefronts x 32)
 constexpr int kTileBytes = kTile * kD * 2;             // 16384: 64 rows of 256 bytes
 constexpr int kOffY = kTileBytes, kOffLse = 2 * kTileBytes, kOffDelta = kOffLse + kTile * 4;
 constexpr int kStageBytes = kOffDelta + kTile * 4;     // X tile, Y tile, lse2 and delta of the streamed rows
@@ -88,7 +90,12 @@ __global__ __launch_bounds__(256) void bwd_prepare(const uint16_t* __restrict__ 
 }
 
 template <bool DQ, bool CAUSAL>
-__global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
+__global__ __launch_bounds__(DQ ? 512 : 256, 1) void bwd_main(const BwdParams p) {
+  // The dQ pass needs half the accumulators of the dK / dV pass and fits two wavefronts per SIMD: its workgroup
+  // is eight wavefronts sharing the streamed K / V tiles.
+  constexpr int kWavesWg = DQ ? 8 : 4;
+  constexpr int kRowsPerWg = kWavesWg * 32;
+  constexpr int kCpy = 16 / kWavesWg;           // copy instructions per wavefront for one 16 KB tile
   __shared__ __attribute__((aligned(16))) unsigned char smem[kSmemBytes];
 
   // Workgroup i runs on XCD i % 8: every XCD gets a contiguous range of (batch, head) pairs.  Under the
@@ -177,10 +184,10 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
   // descriptor's range, and their P / dS are zeroed by index in any case.  lse2 and delta of the 64
   // streamed rows (DQ=false) are copied by the even / odd wavefronts (twice the same bytes: every
   // wavefront then has the same number of copies in flight, which the vmcnt waits rely on).
-  int cvoff[4];
+  int cvoff[kCpy];
 #pragma unroll
-  for (int u = 0; u < 4; ++u) {
-    const int row = 16 * wave + 4 * u + (lane >> 4);
+  for (int u = 0; u < kCpy; ++u) {
+    const int row = 4 * kCpy * wave + 4 * u + (lane >> 4);
     const int chunk = (lane & 15) ^ lds_row_swizzle(row);
     // chunks past the head dimension: an offset that is out of the descriptor's range for every tile, so they
     // arrive as zeros and a tile in LDS always has 128 columns
@@ -192,18 +199,18 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     const int hq = DQ ? 0 : hs * p.group + tile_head(live ? t : 0);
     const int c0 = tile_row0(live ? t : 0);
     const int soff = live ? (int)(((int64_t)c0 * s_ss + (int64_t)hq * s_sh) * 2) : kNoTile;
-    const uint32_t dst = lds_base + stage * kStageBytes + wave * 4096;
+    const uint32_t dst = lds_base + stage * kStageBytes + wave * (kCpy * 1024);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) copy16_to_lds(xrs, dst + u * 1024, cvoff[u], soff);
+    for (int u = 0; u < kCpy; ++u) copy16_to_lds(xrs, dst + u * 1024, cvoff[u], soff);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) copy16_to_lds(yrs, dst + kOffY + u * 1024, cvoff[u], soff);
+    for (int u = 0; u < kCpy; ++u) copy16_to_lds(yrs, dst + kOffY + u * 1024, cvoff[u], soff);
     if (!DQ) {
       const float* src = ((wave & 1) ? p.delta : p.lse2) + ((int64_t)b * p.Hq + hq) * p.Sq;
       copy4_to_lds(rsrc_words(src, (uint32_t)p.Sq * 4u), lds_base + stage * kStageBytes + ((wave & 1) ? kOffDelta : kOffLse),
                    lane * 4, live ? c0 * 4 : kNoTile);
     }
   };
-  constexpr int kCopiesPerTile = DQ ? 8 : 9;
+  constexpr int kCopiesPerTile = DQ ? 2 * kCpy : 2 * kCpy + 1;
   // The same copies one instruction at a time (piece 0 .. kCopiesPerTile - 1), so that the main loop can
   // issue them between MFMAs; the scalar offsets are worked out once per tile by copy_setup.
   int cp_soff = 0, cp_hq = 0, cp_c0 = 0;
@@ -215,9 +222,9 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     cp_soff = cp_live ? (int)(((int64_t)cp_c0 * s_ss + (int64_t)cp_hq * s_sh) * 2) : kNoTile;
   };
   auto copy_piece = [&](int piece, int stage) {
-    const uint32_t dst = lds_base + stage * kStageBytes + wave * 4096;
-    if (piece < 4) copy16_to_lds(xrs, dst + piece * 1024, cvoff[piece], cp_soff);
-    else if (piece < 8) copy16_to_lds(yrs, dst + kOffY + (piece - 4) * 1024, cvoff[piece - 4], cp_soff);
+    const uint32_t dst = lds_base + stage * kStageBytes + wave * (kCpy * 1024);
+    if (piece < kCpy) copy16_to_lds(xrs, dst + piece * 1024, cvoff[piece < kCpy ? piece : 0], cp_soff);
+    else if (piece < 2 * kCpy) copy16_to_lds(yrs, dst + kOffY + (piece - kCpy) * 1024, cvoff[piece < 2 * kCpy ? piece - kCpy : 0], cp_soff);
     else if (!DQ) {
       const float* src = ((wave & 1) ? p.delta : p.lse2) + ((int64_t)b * p.Hq + cp_hq) * p.Sq;
       copy4_to_lds(rsrc_words(src, (uint32_t)p.Sq * 4u), lds_base + stage * kStageBytes + ((wave & 1) ? kOffDelta : kOffLse),
@@ -265,15 +272,16 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
   // wavefront and nobody reads tile t-1 any more, whose stage then receives tile t+3.  Tiles past the end
   // are copied as zeros (and their T1 / T2 computed, unused) so that the number of copies in flight
   // stays the same.
-  constexpr int kDepth = 4;                                // operand reads in flight ahead of the MFMAs (2 and 8 measure the same)
+  // operand reads in flight ahead of the MFMAs (2, 4 and 8 measure the same; 2 keeps the dQ pass inside 256 registers)
+  constexpr int kDepth = DQ ? 2 : 4;
   constexpr int kAcc = DQ ? 8 : 16;                        // slots of an accumulate phase
   constexpr int kP1 = 16, kP2 = 16 + kAcc, kP3 = 32 + kAcc, kSlots = 32 + 2 * kAcc;
   typedef __attribute__((address_space(3))) const bf16x8* lds_bf16x8;
   typedef __attribute__((address_space(3))) const f32x4* lds_f32x4;
   // LDS addresses of the operand reads.  rm_a / tr_a hold, per lane, the addresses inside ONE tile's stage and are
   // moved on to the next stage in place, each at a point of the slot sequence where no read of its kind is due
-  // (rm_a in slots 12-15: the reads of the current tile's T1 / T2 operands are all issued by slot 11 and those of
-  // the next tile start at slot kP2 - kDepth; tr_a in the last kDepth slots, after the last transposed read).
+  // (rm_a in the last kDepth slots of P0: the reads of the current tile's T1 / T2 operands are all issued by then and
+  // those of the next tile start at slot kP2 - kDepth; tr_a in the last kDepth slots, after the last transposed read).
   // ld_cur / ld_next address lse2 / -delta of the current and the next tile.  Everything else about an address
   // is an immediate offset of the LDS instruction.
   int rm_a[8], tr_a[4][2];
@@ -391,7 +399,7 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
     if (s < kP3) return read_rm(0, s - kP2);
     return read_acc(1, s - kP3);
   };
-  static_assert(kP2 - kDepth >= 16 && kP1 - kDepth <= 12, "rm_a moves in slots 12-15");
+  static_assert(kP2 - kDepth >= 16 && 4 % kDepth == 0, "rm_a moves in the last kDepth slots of P0, tr_a in the last kDepth slots of P3");
 
   if (ntiles > 0) {
     copy_tile(0, 0);
@@ -420,17 +428,19 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
         yf[ks] = bf16x8{};
       }
     }
-    // Pin the loads here (the copies are invisible to the compiler's wait counting), the MFMA operands into
-    // accumulation registers: the arithmetic registers are needed for the tiles of T1 / T2 that the vector
-    // unit works on.
+    // Pin the loads here (the copies are invisible to the compiler's wait counting).  The dK / dV pass keeps these
+    // MFMA operands in accumulation registers: its arithmetic registers are needed for the tiles of T1 / T2 that
+    // the vector unit works on.  The dQ pass at two wavefronts per SIMD uses no accumulation registers at all (a
+    // kernel that does gets its 256 registers split 128 / 128).
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) { asm volatile("" : "+a"(xf[ks])); asm volatile("" : "+a"(yf[ks])); }
+    for (int ks = 0; ks < 8; ++ks) {
+      if (DQ) { asm volatile("" : "+v"(xf[ks])); asm volatile("" : "+v"(yf[ks])); }
+      else { asm volatile("" : "+a"(xf[ks])); asm volatile("" : "+a"(yf[ks])); }
+    }
     asm volatile("" : "+v"(lse2_lane), "+v"(delta_lane));
   }
   if (ntiles > 0) {
-    if (DQ) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
-    static_assert(kCopiesPerTile == (DQ ? 8 : 9), "the vmcnt immediates are one and two tiles of copies");
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * kCopiesPerTile) : "memory");      // two tiles of copies may stay in flight
     __builtin_amdgcn_s_barrier();
     if (DQ) {
 #pragma unroll
@@ -457,8 +467,7 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
   }
   for (int t = 0; t < ntiles; ++t) {
     const int c0 = tile_row0(t);
-    if (DQ) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kCopiesPerTile) : "memory");          // one tile of copies stays in flight
     __builtin_amdgcn_s_barrier();
     copy_setup(t + 3);
     // byte distance from this tile's stage to the next tile's, and from that one to the one after
@@ -472,7 +481,10 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
       vector_slot(i, ta1, ta2, 0);
       if (i < kCopiesPerTile) copy_piece(i, (t + 3) & 3);
       ring[i % kDepth] = read_slot(i + kDepth);
-      if (i >= 12) { rm_a[2 * (i - 12)] += step1; rm_a[2 * (i - 12) + 1] += step1; }      // on to the next tile
+      if (i >= 16 - kDepth) {                            // the last read of this tile's T1 / T2 operands is out: on to the next
+#pragma unroll
+        for (int j = 0; j < 8 / kDepth; ++j) rm_a[(i - (16 - kDepth)) * (8 / kDepth) + j] += step1;
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
@@ -502,8 +514,11 @@ __global__ __launch_bounds__(256, 1) void bwd_main(const BwdParams p) {
       if (!DQ && i >= 8 && i < 12) read_nd(true, 1, i - 8);            // T2 of (t+1, second half): P0 of the next tile
       ring[(kP3 + i) % kDepth] = read_slot(kP3 + i + kDepth);
       if (i >= kAcc - kDepth) {                          // the last transposed read of this tile has been issued
-        const int db = i - (kAcc - kDepth);
-        tr_a[db][0] += step1; tr_a[db][1] += step1;
+#pragma unroll
+        for (int j = 0; j < 4 / kDepth; ++j) {
+          const int db = (i - (kAcc - kDepth)) * (4 / kDepth) + j;
+          tr_a[db][0] += step1; tr_a[db][1] += step1;
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -666,16 +681,16 @@ int bwd_block(const void* dout, const void* q, const void* k, const void* v,
                        static_cast<const uint16_t*>(dout), static_cast<const uint16_t*>(out), lse,
                        delta_buf, lse2_buf, softmax_d, B, Sq, Hq, D, q_sb, q_ss, q_sh, o_sb, o_ss, o_sh);
     // dQ: one workgroup per 128 query rows
-    p.n_tiles = (Sq + kRowsPerWg - 1) / kRowsPerWg;
+    p.n_tiles = (Sq + kRowsQ - 1) / kRowsQ;
     p.total = B * Hq * p.n_tiles;
     p.per_xcd = (p.total + 7) / 8;
     p.heads_per_xcd = (B * Hq) % 8 == 0 ? (B * Hq) / 8 : 0;
-    if (causal) hipLaunchKernelGGL((bwd_main<true, true>), dim3(p.per_xcd * 8), dim3(256), 0, st, p);
-    else hipLaunchKernelGGL((bwd_main<true, false>), dim3(p.per_xcd * 8), dim3(256), 0, st, p);
+    if (causal) hipLaunchKernelGGL((bwd_main<true, true>), dim3(p.per_xcd * 8), dim3(512), 0, st, p);
+    else hipLaunchKernelGGL((bwd_main<true, false>), dim3(p.per_xcd * 8), dim3(512), 0, st, p);
   }
   if (Sc > 0) {
     // dK, dV: one workgroup per 128 keys of one kv head
-    p.n_tiles = (Sc + kRowsPerWg - 1) / kRowsPerWg;
+    p.n_tiles = (Sc + kRowsKv - 1) / kRowsKv;
     p.total = B * Hkv * p.n_tiles;
     p.per_xcd = (p.total + 7) / 8;
     p.heads_per_xcd = (B * Hkv) % 8 == 0 ? (B * Hkv) / 8 : 0;
