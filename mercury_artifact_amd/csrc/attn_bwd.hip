@@ -213,23 +213,29 @@ __global__ __launch_bounds__(DQ ? 512 : 256, 1) void bwd_main(const BwdParams p)
   constexpr int kCopiesPerTile = DQ ? 2 * kCpy : 2 * kCpy + 1;
   // The same copies one instruction at a time (piece 0 .. kCopiesPerTile - 1), so that the main loop can
   // issue them between MFMAs; the scalar offsets are worked out once per tile by copy_setup.
-  int cp_soff = 0, cp_hq = 0, cp_c0 = 0;
-  bool cp_live = false;
-  auto copy_setup = [&](int t) {
-    cp_live = t < ntiles;
-    cp_hq = DQ ? 0 : hs * p.group + tile_head(cp_live ? t : 0);
-    cp_c0 = tile_row0(cp_live ? t : 0);
-    cp_soff = cp_live ? (int)(((int64_t)cp_c0 * s_ss + (int64_t)cp_hq * s_sh) * 2) : kNoTile;
+  // Which tile comes three tiles ahead is kept as a pair of running counters (position inside the head's span,
+  // head of the group) instead of a division per tile: every scalar instruction of the loop takes an issue slot of
+  // the one wavefront a SIMD runs in the dK / dV pass.
+  int cp_soff = 0, cp_ld_soff = 0;
+  int nx_r = DQ ? 3 : (span > 0 ? 3 % span : 0), nx_h = DQ ? 0 : (span > 0 ? 3 / span : 0);
+  const uint32_t ld_rows = (uint32_t)p.B * (uint32_t)p.Hq * (uint32_t)p.Sq;     // the host keeps this below 2^30
+  const u32x4 ldrs = rsrc_words((wave & 1) ? p.delta : p.lse2, ld_rows * 4u);
+  auto copy_setup = [&]() {
+    const bool live = DQ ? nx_r < span : nx_h < heads_str;
+    const uint32_t hq = DQ ? 0u : (uint32_t)(hs * p.group + (live ? nx_h : 0));
+    const uint32_t c0 = (uint32_t)((first_tile + (live ? nx_r : 0)) * kTile);
+    // element offsets stay below 2^31 (checked by the host), so 32-bit arithmetic is exact
+    cp_soff = live ? (int)((c0 * (uint32_t)s_ss + hq * (uint32_t)s_sh) * 2u) : kNoTile;
+    if (!DQ) cp_ld_soff = live ? (int)((((uint32_t)b * (uint32_t)p.Hq + hq) * (uint32_t)p.Sq + c0) * 4u) : kNoTile;
+    ++nx_r;
+    if (!DQ && nx_r == span) { nx_r = 0; ++nx_h; }
   };
   auto copy_piece = [&](int piece, int stage) {
     const uint32_t dst = lds_base + stage * kStageBytes + wave * (kCpy * 1024);
     if (piece < kCpy) copy16_to_lds(xrs, dst + piece * 1024, cvoff[piece < kCpy ? piece : 0], cp_soff);
     else if (piece < 2 * kCpy) copy16_to_lds(yrs, dst + kOffY + (piece - kCpy) * 1024, cvoff[piece < 2 * kCpy ? piece - kCpy : 0], cp_soff);
-    else if (!DQ) {
-      const float* src = ((wave & 1) ? p.delta : p.lse2) + ((int64_t)b * p.Hq + cp_hq) * p.Sq;
-      copy4_to_lds(rsrc_words(src, (uint32_t)p.Sq * 4u), lds_base + stage * kStageBytes + ((wave & 1) ? kOffDelta : kOffLse),
-                   lane * 4, cp_live ? cp_c0 * 4 : kNoTile);
-    }
+    else if (!DQ)
+      copy4_to_lds(ldrs, lds_base + stage * kStageBytes + ((wave & 1) ? kOffDelta : kOffLse), lane * 4, cp_ld_soff);
   };
 
   // row-major operand reads (A of T1 / T2): lane (ln, hf) reads chunk 2 kk + hf of row 32 mb + ln
@@ -465,11 +471,13 @@ __global__ __launch_bounds__(DQ ? 512 : 256, 1) void bwd_main(const BwdParams p)
       for (int g = 0; g < 4; ++g) read_nd(false, 1, g);        // for T2 of the second half, first thing in the loop
     }
   }
+  int cur_r = 0;                                         // t % span
   for (int t = 0; t < ntiles; ++t) {
-    const int c0 = tile_row0(t);
+    const int c0 = (first_tile + cur_r) * kTile;
+    if (++cur_r == span) cur_r = 0;                      // (t + 1) % span
     asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kCopiesPerTile) : "memory");          // one tile of copies stays in flight
     __builtin_amdgcn_s_barrier();
-    copy_setup(t + 3);
+    copy_setup();
     // byte distance from this tile's stage to the next tile's, and from that one to the one after
     const int step1 = ((t + 1) & 3) == 0 ? -3 * kStageBytes : kStageBytes;
     const int step2 = ((t + 2) & 3) == 0 ? -3 * kStageBytes : kStageBytes;
@@ -647,6 +655,7 @@ int bwd_block(const void* dout, const void* q, const void* k, const void* v,
   const int64_t q_span = ((int64_t)Sq * q_ss + (int64_t)Hq * q_sh) * 2;
   const int64_t k_span = (int64_t)Sc * k_ss * 2;
   if (q_span >= (int64_t(1) << 31) || k_span >= (int64_t(1) << 31)) return MHIP_EUNSUPPORTED;
+  if ((int64_t)B * Hq * Sq >= (int64_t(1) << 30)) return MHIP_EUNSUPPORTED;     // lse2 / delta are addressed with 32-bit byte offsets
   // below 128 the lanes of the missing columns carry the offset kNoColumn, which has to be out of range
   if (D < kD && (q_span >= (int64_t(1) << 30) || k_span >= (int64_t(1) << 30))) return MHIP_EUNSUPPORTED;
   if (own_scratch && Sq > 0) {
