@@ -330,6 +330,7 @@ class LocalMesh:
         self._lock = threading.Lock()
         self._gathers = {}
         self._world_barrier = threading.Barrier(self.world)
+        self._failed = threading.Event()          # set by the first rank that raises: the others stop waiting
         mesh = self
 
         class _Dist:
@@ -384,7 +385,11 @@ class LocalMesh:
         re-raises the first exception of any rank."""
         ranks = list(range(self.world)) if ranks is None else list(ranks)
         results = {}
-        errors = {}
+        errors = []                                # (rank, exception) in the order they happened
+        # a fresh start: nothing of an earlier run (undelivered messages, barriers a failure broke) is left over
+        self._failed.clear()
+        self._mail, self._gathers = {}, {}
+        self._world_barrier = threading.Barrier(self.world)
         device = torch.cuda.current_device() if torch.cuda.is_available() else None
         stream = torch.cuda.current_stream() if torch.cuda.is_available() else None
 
@@ -398,7 +403,9 @@ class LocalMesh:
                 else:
                     results[r] = fn(r)
             except BaseException as exc:          # noqa: BLE001 -- handed to the caller below
-                errors[r] = exc
+                with self._lock:
+                    errors.append((r, exc))
+                self._failed.set()
                 for slot in list(self._gathers.values()):
                     slot["barrier"].abort()
                 self._world_barrier.abort()
@@ -415,10 +422,14 @@ class LocalMesh:
         finally:
             _ACTIVE_MESH[0] = None
         if errors:
-            first = min(errors)
-            real = [r for r in sorted(errors) if not isinstance(errors[r], threading.BrokenBarrierError)]
-            raise errors[real[0] if real else first]
+            # the first thing that went wrong, not what the other ranks ran into because of it
+            own = [exc for _, exc in errors if not isinstance(exc, (threading.BrokenBarrierError, _PeerFailed))]
+            raise own[0] if own else errors[0][1]
         return [results[r] for r in ranks]
+
+
+class _PeerFailed(RuntimeError):
+    """Raised in a rank that was waiting for a message when another rank of the mesh failed."""
 
 
 class _MeshSendRecv:
@@ -448,10 +459,17 @@ class _MeshSendRecv:
             raise RuntimeError("wait called before commit")
         me = self._mesh.rank()
         for _, from_rank, _, res in self._ops:
-            try:
-                got = self._mesh._box(from_rank, me).get(timeout=self._mesh.timeout)
-            except queue.Empty:
-                raise RuntimeError(f"rank {me} waited {self._mesh.timeout} s for a message from rank {from_rank}") from None
+            box, waited, got = self._mesh._box(from_rank, me), 0.0, None
+            while got is None:
+                if self._mesh._failed.is_set():
+                    raise _PeerFailed(f"rank {me} stopped waiting for rank {from_rank}: another rank raised")
+                try:
+                    got = box.get(timeout=0.05)
+                except queue.Empty:
+                    waited += 0.05
+                    if waited >= self._mesh.timeout:
+                        raise RuntimeError(f"rank {me} waited {self._mesh.timeout} s for a message from rank "
+                                           f"{from_rank}") from None
             res.copy_(got)
         self._committed = False
         self._ops = []

@@ -261,3 +261,38 @@ def test_local_mesh_replays_the_ring_protocol_of_all_ranks():
 
     with pytest.raises(RuntimeError, match="waited"):
         small.run(starved)
+
+
+def test_local_mesh_reports_the_first_failure_and_releases_the_waiting_ranks():
+    """A rank that raises ends the whole run at once: the ranks waiting for its messages stop waiting (they do not sit
+    out the time limit), and what run() raises is that rank's own exception, whichever rank index it had."""
+    import time
+
+    import mercury_artifact_amd as M
+
+    mesh = M.LocalMesh((4,), timeout=30.0)
+
+    def rank_fn(r):
+        comm = mesh.SendRecv()
+        if r == 3:
+            time.sleep(0.2)                      # the others are waiting by now
+            raise ValueError("rank 3 broke")
+        comm.send_recv((r + 1) % 4, (r - 1) % 4, torch.zeros(1))
+        comm.commit()
+        comm.wait()                              # rank 0 waits for rank 3, which never sends
+        return r
+
+    begin = time.monotonic()
+    with pytest.raises(ValueError, match="rank 3 broke"):
+        mesh.run(rank_fn)
+    assert time.monotonic() - begin < 5.0
+    # the mesh is usable again afterwards: the messages of the failed run are gone, the barrier works
+    def again(r):
+        comm = mesh.SendRecv()
+        got = comm.send_recv((r + 1) % 4, (r - 1) % 4, torch.full((1,), float(r + 10)))
+        comm.commit()
+        comm.wait()
+        mesh.dist.barrier()
+        return int(got.item())
+
+    assert mesh.run(again) == [13, 10, 11, 12]
