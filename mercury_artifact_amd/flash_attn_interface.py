@@ -24,7 +24,7 @@ def _strides3(t: torch.Tensor):
     return t.stride(0), t.stride(1), t.stride(2)
 
 
-def _check_block_inputs(q, k, v, dropout_p, window_size_left, window_size_right, softcap, alibi_slopes):
+def _check_block_inputs(q, k, v, dropout_p, window_size_left, window_size_right, softcap, alibi_slopes, causal=False):
     N.require_cuda(q, k, v)
     if dropout_p not in (0, 0.0, None):
         raise RuntimeError("dropout_p != 0 is not supported (the ring templates always pass 0)")
@@ -32,8 +32,9 @@ def _check_block_inputs(q, k, v, dropout_p, window_size_left, window_size_right,
         raise RuntimeError("softcap != 0 is not supported")
     if alibi_slopes is not None:
         raise RuntimeError("alibi_slopes is not supported")
-    if (window_size_left not in (-1, None)) or (window_size_right not in (-1, 0, None)):
-        raise RuntimeError("sliding windows are not supported (window_size must be (-1, -1))")
+    # a right window of 0 is how flash-attn spells the causal mask; without `causal` it would be a mask of its own
+    if (window_size_left not in (-1, None)) or (window_size_right not in ((-1, 0, None) if causal else (-1, None))):
+        raise RuntimeError("sliding windows are not supported (window_size must be (-1, -1), or (-1, 0) with causal=True)")
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise RuntimeError("q, k, v must be (batch, seq, heads, head_dim)")
     if q.stride(-1) != 1 or k.stride(-1) != 1 or v.stride(-1) != 1:
@@ -128,7 +129,7 @@ def _flash_attn_forward(
     """Returns ``(out, softmax_lse, S_dmask, rng_state)``; the last two are empty placeholders
     (no dropout), kept because the generated code asserts ``len(outputs) == 4``
     (utils/flash_attn_dsl.py:175)."""
-    _check_block_inputs(q, k, v, dropout_p, window_size_left, window_size_right, softcap, alibi_slopes)
+    _check_block_inputs(q, k, v, dropout_p, window_size_left, window_size_right, softcap, alibi_slopes, causal)
     out, lse = attn_fwd_block(q, k, v, softmax_scale, bool(causal), q_descale, k_descale, v_descale)
     empty = torch.empty((0,), dtype=q.dtype if q.dtype == torch.bfloat16 else torch.bfloat16, device=q.device)
     rng = torch.empty((2,), dtype=torch.int64, device=q.device)
@@ -227,6 +228,6 @@ def _flash_attn_backward(
     """Keyword surface of utils/attn_bwd_dsl.py:86-115; dq/dk/dv are caller-allocated
     (``torch.empty``, utils/attn_bwd_dsl.py:83-84) and every element of them is written.
     Returns ``softmax_d`` (rowsum(dout * out), (B,Hq,Sq) fp32) like flash-attn does."""
-    _check_block_inputs(q, k, v, dropout_p, window_size_left, window_size_right, softcap, alibi_slopes)
+    _check_block_inputs(q, k, v, dropout_p, window_size_left, window_size_right, softcap, alibi_slopes, causal)
     return attn_bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_scale, bool(causal),
                           bool(deterministic))

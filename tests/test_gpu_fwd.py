@@ -310,3 +310,31 @@ def test_config0_through_the_gpu_path():
             M.flash_attn_pack_kv(qd, dev[rank], o, lse, scale, ring=M.LocalRing((4,), rank, dev),
                                  deferred_merge=deferred, fused_epilogue=deferred)
             _check(o, lse, ref_o, ref_l, f"config0 rank {rank} deferred={deferred}")
+
+
+def test_block_operators_refuse_what_the_kernels_do_not_implement():
+    """flash-attn arguments the ring templates never set (utils/flash_attn_dsl.py:159-173 passes dropout 0, no alibi,
+    the window it was given, softcap 0): anything else is an error here, never a silently different result.  A right
+    window of 0 is flash-attn's spelling of the causal mask and is accepted only together with ``causal``."""
+    import mercury_artifact_amd as M
+
+    B, S, H, D = 1, 64, 1, 128
+    q = torch.randn(B, S, H, D, device="cuda").bfloat16()
+    k, v = torch.randn_like(q), torch.randn_like(q)
+    base = dict(q=q, k=k, v=v, dropout_p=0.0, softmax_scale=D ** -0.5, causal=False, window_size_left=-1,
+                window_size_right=-1, softcap=0.0, alibi_slopes=None, return_softmax=False)
+    M._flash_attn_forward(**base)
+    M._flash_attn_forward(**dict(base, causal=True, window_size_right=0))
+    for change in (dict(window_size_right=0), dict(window_size_left=16), dict(window_size_right=8, causal=True),
+                   dict(dropout_p=0.1), dict(softcap=30.0), dict(alibi_slopes=torch.ones(H, device="cuda"))):
+        with pytest.raises(RuntimeError, match="not supported"):
+            M._flash_attn_forward(**dict(base, **change))
+    out, lse = M.attn_fwd_block(q, k, v, D ** -0.5)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    back = dict(dout=q, q=q, k=k, v=v, out=out, softmax_lse=lse, dq=dq, dk=dk, dv=dv, dropout_p=0.0,
+                softmax_scale=D ** -0.5, causal=False, window_size_left=-1, window_size_right=-1, softcap=0.0,
+                alibi_slopes=None, deterministic=False, rng_state=None)
+    M._flash_attn_backward(**back)
+    for change in (dict(window_size_right=0), dict(window_size_left=16), dict(dropout_p=0.1), dict(softcap=30.0)):
+        with pytest.raises(RuntimeError, match="not supported"):
+            M._flash_attn_backward(**dict(back, **change))
