@@ -103,8 +103,9 @@ def _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, 
     ``two_streams`` (with the deferred fold only, where the block launches do not depend on each other): every
     other block launch goes to a second stream, so that the tail of one launch (workgroups of its last round,
     drained pipelines) overlaps the head of the next; the fold waits for both.  The side stream starts behind
-    everything queued on the current stream when the step begins; a multi-GPU ring would make it wait for the
-    hop's completion event instead."""
+    everything queued on the current stream when the step begins, and a block launched there waits for the event
+    recorded on the current stream right behind the hop that delivers its chunk (so for the hop's copy, not for the
+    block launch that follows it on the current stream)."""
     blocks = []
     _out = None
     _lse = None
@@ -127,6 +128,7 @@ def _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, 
                       "(same result, one pass over the fp32 accumulator per block)", RuntimeWarning, stacklevel=3)
     done = 0
     main = side = None
+    kv_ready = next_ready = None
     if two_streams and defer:
         main = torch.cuda.current_stream(q.device)
         side = _side_stream(q.device)
@@ -138,17 +140,29 @@ def _ring_forward(q, kv, o, lse, softmax_scale, dropout_p, causal, window_size, 
         for step, hop in enumerate(steps):
             if step == 0:
                 _kv = kv[:, :, rows].contiguous()
+                kv_ready = None
+                if side is not None and part > 0:      # the sub-chunk copy above sits behind earlier launches
+                    kv_ready = torch.cuda.Event()
+                    kv_ready.record(main)
             else:
                 part_ring.wait()
                 _kv = _next_kv
+                kv_ready = next_ready
             if hop is not None:
                 send_to, recv_from = _neighbours(part_ring, hop)
                 _next_kv = part_ring.send_recv(send_to, recv_from, _kv)
                 part_ring.commit()
+                next_ready = None
+                if side is not None:                   # what the hop enqueued on the current stream ends here
+                    next_ready = torch.cuda.Event()
+                    next_ready.record(main)
             _k = _kv[0]
             _v = _kv[1]
             params = _fwd_params(q, _k, _v, softmax_scale, dropout_p, causal, window_size, alibi_slopes, **extra)
             if side is not None and done % 2 == 1:
+                if kv_ready is not None:
+                    side.wait_event(kv_ready)
+                _kv.record_stream(side)              # may have been allocated by the hop on the current stream
                 with torch.cuda.stream(side):
                     outputs = _flash_attn_forward(**params)
                 for t in outputs[:2]:

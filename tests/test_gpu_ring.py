@@ -242,3 +242,34 @@ def test_reduce_buffer_ring_all_ranks(mesh):
     torch.cuda.synchronize()
     for r in range(W):
         _compare(outs[r], lses[r], ref_o[:, r * Sc:(r + 1) * Sc], ref_l[:, :, r * Sc:(r + 1) * Sc])
+
+
+@pytest.mark.parametrize("copy", [False, True])
+@pytest.mark.parametrize("ring_divide", [1, 2])
+def test_two_stream_step_is_bit_identical(copy, ring_divide):
+    """``two_streams=True`` sends every other block launch to a second stream.  Same kernels on the same operands,
+    one fold: the step has to give the single-stream result bit for bit, also when the hops copy the chunks (a block on
+    the second stream then has to wait for the copy that delivers its chunk) and with sub-chunk loops; repeated, so
+    that a launch that ran ahead of its operand would show."""
+    import mercury_artifact_amd as M
+
+    B, S, H, D, W, rank = 1, 512, 4, 128, 4, 1
+    g = torch.Generator(device="cuda").manual_seed(17)
+    q = torch.randn(B, S, H, D, generator=g, device="cuda").bfloat16()
+    kvs = [torch.randn(2, B, S, H, D, generator=g, device="cuda").bfloat16() for _ in range(W)]
+    scale = D ** -0.5
+
+    def step(two):
+        o = torch.empty_like(q)
+        lse = torch.empty(B, H, S, dtype=torch.float32, device="cuda")
+        M.flash_attn_pack_kv(q, kvs[rank], o, lse, scale, ring=M.LocalRing((W,), rank, kvs, copy=copy),
+                             ring_divide=ring_divide, two_streams=two)
+        return o, lse
+
+    ref_o, ref_l = step(False)
+    for _ in range(5):
+        o, lse = step(True)
+        torch.cuda.synchronize()
+        assert torch.equal(o, ref_o) and torch.equal(lse, ref_l)
+    ro, rl = O.ring_forward(q.float().cpu(), [c.float().cpu() for c in kvs], O.single_ring_order(rank, W), scale)
+    assert (ref_o.float().cpu() - ro).abs().max().item() <= 2e-2
