@@ -4,14 +4,15 @@
 //     P = exp(scale * q k^T - lse),  delta = rowsum(dout * out)
 //     dV = P^T dout,  dP = dout v^T,  dS = P * (dP - delta),  dQ = scale * dS k,  dK = scale * dS^T q
 //
-// Three kernels, no atomics (so every run is deterministic):
-//   bwd_prepare  delta[b,h,i] = sum_d dout * out and lse2 = lse * log2(e), with -inf (a row that saw no
-//                key) turned into +inf so that P = exp2(s - lse2) = 0 there       (bandwidth bound)
-//   bwd_main<DQ=false>  one workgroup per 128 keys of one KV head: K and V rows stay in registers,
-//                Q / dout tiles of the (grouped) query heads stream through LDS; accumulates dK, dV
+// Two kernels, launched in this order, no atomics (so every run is deterministic):
 //   bwd_main<DQ=true>   one workgroup per 256 query rows of one head (eight wavefronts, two per SIMD: this pass
 //                has half the accumulators of the other and fits 256 registers): Q and dout rows stay in
-//                registers, K / V tiles stream through LDS; accumulates dQ
+//                registers, K / V tiles stream through LDS; accumulates dQ.  Its prologue also works out, per
+//                query row, delta = sum_d dout * out and lse2 = lse * log2(e) (with -inf, a row that saw no key,
+//                turned into +inf so that P = exp2(s - lse2) = 0 there) and leaves them in the workspace
+//   bwd_main<DQ=false>  one workgroup per 128 keys of one KV head: K and V rows stay in registers,
+//                Q / dout tiles of the (grouped) query heads stream through LDS together with their lse2 /
+//                delta from the workspace; accumulates dK, dV
 // Both instances share one body.  "Stationary" rows (32 per wavefront) sit in the lane index of every
 // MFMA accumulator, "streamed" rows in its registers, exactly as in the forward kernel:
 //     T1[c][r] = X_str[c] . X_st[r]      (scores)          T2[c][r] = Y_str[c] . Y_st[r]      (dP)
@@ -45,7 +46,9 @@ constexpr int kNoColumn = 0x7fff0000; // vector offset with the same effect for 
 
 struct BwdParams {
   const uint16_t* q; const uint16_t* k; const uint16_t* v; const uint16_t* dout;
-  const float* lse2; const float* delta;   // both (B, Hq, Sq) fp32, written by bwd_prepare
+  const uint16_t* out; const float* lse;   // saved output and log-sum-exp of the forward
+  float* lse2; float* delta;               // both (B, Hq, Sq) fp32: written by the dQ pass, read by the dK / dV pass
+  float* softmax_d;                        // rowsum(dout * out) itself for the caller, or null
   uint16_t* dq; uint16_t* dk; uint16_t* dv; float* dq_acc;
   int B, Sq, Sc, Hq, Hkv, group;
   int D;            // head dimension of the tensors, a multiple of 8 up to kD; columns D .. kD-1 are zeros on chip
@@ -56,38 +59,6 @@ struct BwdParams {
   int per_xcd;
   int heads_per_xcd;   // (batch, stationary head) pairs per XCD when they divide evenly, else 0
 };
-
-// delta = rowsum(dout * out): one row of D <= 128 values per 16 lanes (8 values each); lse2 as described above
-__global__ __launch_bounds__(256) void bwd_prepare(const uint16_t* __restrict__ dout, const uint16_t* __restrict__ out,
-                                                   const float* __restrict__ lse, float* __restrict__ delta,
-                                                   float* __restrict__ lse2, float* __restrict__ softmax_d,
-                                                   int B, int Sq, int Hq, int D,
-                                                   int64_t sb, int64_t ss, int64_t sh,
-                                                   int64_t o_sb, int64_t o_ss, int64_t o_sh) {
-  const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
-  const int64_t rows = (int64_t)B * Hq * Sq;
-  const int c = threadIdx.x & 15;
-  float acc = 0.f;
-  if (row < rows && c * 8 < D) {
-    const int s = (int)(row % Sq);
-    const int64_t bh = row / Sq;
-    const int h = (int)(bh % Hq);
-    const int b = (int)(bh / Hq);
-    const int64_t off = b * sb + (int64_t)s * ss + h * sh + c * 8;
-    const u32x4 a = *reinterpret_cast<const u32x4*>(dout + off);
-    const u32x4 o = *reinterpret_cast<const u32x4*>(out + (b * o_sb + (int64_t)s * o_ss + h * o_sh + c * 8));
-#pragma unroll
-    for (int j = 0; j < 4; ++j) acc += bf16_lo(a[j]) * bf16_lo(o[j]) + bf16_hi(a[j]) * bf16_hi(o[j]);
-  }
-#pragma unroll
-  for (int m = 8; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 16);
-  if (row < rows && c == 0) {      // (B, Hq, Sq) contiguous
-    delta[row] = -acc;       // stored negated: the main kernels start dP^T = Y Z^T from it (C operand of the first MFMA)
-    if (softmax_d) softmax_d[row] = acc;     // the value itself, for callers that want flash-attn's softmax_d back
-    const float l = lse[row];
-    lse2[row] = (l == -INFINITY) ? INFINITY : l * kLog2e;
-  }
-}
 
 template <bool DQ, bool CAUSAL>
 __global__ __launch_bounds__(DQ ? 512 : 256, 1) void bwd_main(const BwdParams p) {
@@ -418,8 +389,6 @@ __global__ __launch_bounds__(DQ ? 512 : 256, 1) void bwd_main(const BwdParams p)
     if (DQ) {
       const int64_t off = b * p.q_sb + (int64_t)row * p.q_ss + hs * p.q_sh + hf * 8;
       xp = p.q + off; yp = p.dout + off;
-      lse2_lane = p.lse2[((int64_t)b * p.Hq + hs) * p.Sq + row];
-      delta_lane = p.delta[((int64_t)b * p.Hq + hs) * p.Sq + row];
     } else {
       const int64_t off = b * p.k_sb + (int64_t)row * p.k_ss + hs * p.k_sh + hf * 8;
       xp = p.k + off; yp = p.v + off;
@@ -442,6 +411,32 @@ __global__ __launch_bounds__(DQ ? 512 : 256, 1) void bwd_main(const BwdParams p)
     for (int ks = 0; ks < 8; ++ks) {
       if (DQ) { asm volatile("" : "+v"(xf[ks])); asm volatile("" : "+v"(yf[ks])); }
       else { asm volatile("" : "+a"(xf[ks])); asm volatile("" : "+a"(yf[ks])); }
+    }
+    if (DQ) {
+      // This pass runs first and prepares what both passes need per query row: delta = rowsum(dout * out), kept
+      // negated (the dP products start from it), and lse2 = lse * log2(e) with -inf (a row that saw no key) turned
+      // into +inf so that P = exp2(s - lse2) = 0 there.  The lane pair (l, l ^ 32) holds the two halves of the
+      // row's dout; the matching halves of out are read here once.
+      const uint16_t* op = p.out + b * p.o_sb + (int64_t)row * p.o_ss + hs * p.o_sh + hf * 8;
+      float part = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        if (ks * 16 + hf * 8 < p.D) {
+          const bf16x8 o8 = *reinterpret_cast<const bf16x8*>(op + ks * 16);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) part = __builtin_fmaf((float)yf[ks][j], (float)o8[j], part);
+        }
+      }
+      const float delta = pair_sum(part);
+      const int64_t r = ((int64_t)b * p.Hq + hs) * p.Sq + row;
+      const float l = p.lse[r];
+      lse2_lane = (l == -INFINITY) ? INFINITY : l * kLog2e;
+      delta_lane = -delta;
+      if (hf == 0 && my_r < n_st) {
+        p.delta[r] = delta_lane;
+        p.lse2[r] = lse2_lane;
+        if (p.softmax_d) p.softmax_d[r] = delta;     // for callers that want flash-attn's softmax_d back
+      }
     }
     asm volatile("" : "+v"(lse2_lane), "+v"(delta_lane));
   }
@@ -671,7 +666,8 @@ int bwd_block(const void* dout, const void* q, const void* k, const void* v,
   const int64_t slot = ((int64_t)B * Hq * Sq + 3) & ~int64_t(3);                // 16-byte aligned
   float* lse2_buf = delta_buf + slot;
   float* softmax_d = own_scratch ? nullptr : lse2_buf + slot;      // the built-in scratch has no room for it
-  p.lse2 = lse2_buf; p.delta = delta_buf;
+  p.lse2 = lse2_buf; p.delta = delta_buf; p.softmax_d = softmax_d;
+  p.out = static_cast<const uint16_t*>(out); p.lse = lse;
   p.dq = static_cast<uint16_t*>(dq); p.dk = static_cast<uint16_t*>(dk); p.dv = static_cast<uint16_t*>(dv);
   p.dq_acc = dq_acc;
   p.B = B; p.Sq = Sq; p.Sc = Sc; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv;
@@ -685,11 +681,7 @@ int bwd_block(const void* dout, const void* q, const void* k, const void* v,
   const bool causal = mask == MHIP_MASK_CAUSAL;
 
   if (Sq > 0) {
-    const int64_t rows = (int64_t)B * Hq * Sq;
-    hipLaunchKernelGGL(bwd_prepare, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
-                       static_cast<const uint16_t*>(dout), static_cast<const uint16_t*>(out), lse,
-                       delta_buf, lse2_buf, softmax_d, B, Sq, Hq, D, q_sb, q_ss, q_sh, o_sb, o_ss, o_sh);
-    // dQ: one workgroup per 128 query rows
+    // dQ (and delta / lse2 for both passes): one workgroup per 256 query rows; has to run before the dK / dV pass
     p.n_tiles = (Sq + kRowsQ - 1) / kRowsQ;
     p.total = B * Hq * p.n_tiles;
     p.per_xcd = (p.total + 7) / 8;
@@ -747,7 +739,7 @@ extern "C" int mhip_attn_bwd_block_noalloc(const void* dout, const void* q, cons
                                            int64_t o_sb, int64_t o_ss, int64_t o_sh,
                                            float softmax_scale, int mask, int deterministic, void* stream) {
   (void)deterministic;
-  // bwd_prepare overwrites the part of the scratch the two main kernels read, so nothing has to be cleared
+  // the dQ pass overwrites the part of the scratch the dK / dV pass reads, so nothing has to be cleared
   return bwd_block(dout, q, k, v, out, lse, dq, dk, dv, dq_acc, B, Sq, Sc, Hq, Hkv, D, q_sb, q_ss, q_sh,
                    k_sb, k_ss, k_sh, dk_sb, dk_ss, dk_sh, dq_sb, dq_ss, dq_sh, o_sb, o_ss, o_sh, softmax_scale, mask,
                    nullptr, true,
