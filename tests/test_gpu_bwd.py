@@ -49,6 +49,8 @@ BWD_SHAPES = [
     (1, 700, 64, 3, 1, False),       # many rows of three grouped heads, few keys
     (1, 1, 2, 1, 1, False),          # a single query row (with one key every gradient of q is exactly zero)
     (2, 384, 384, 8, 4, True),       # causal with B*Hq and B*Hkv multiples of 8: the per-XCD longest-first order
+    (1, 1100, 900, 2, 2, False),     # five 256-row workgroups of the dQ pass, the last one ragged; 15 key tiles
+    (1, 900, 1100, 2, 1, True),      # the same under the causal mask with more keys than rows, grouped heads
 ]
 
 
