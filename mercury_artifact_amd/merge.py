@@ -21,23 +21,25 @@ __all__ = ["get_default_args", "update_out_and_lse", "_update_out_and_lse", "fla
 
 
 @cache
-def _get_default_args(func):
-    spec = inspect.getfullargspec(func)
-    defaults = spec.defaults if spec.defaults is not None else ()
-    padded = (None,) * (len(spec.args) - len(defaults)) + tuple(defaults)
-    args = dict(zip(spec.args, padded))
-    if "softcap" in args:
-        args["softcap"] = 0.0
-    return args
+def _keyword_defaults(func):
+    """Name -> default of every parameter that can be passed by keyword position-or-name; ``None`` where the
+    signature gives no default; ``softcap`` pinned to 0.0."""
+    named = (inspect.Parameter.POSITIONAL_ONLY, inspect.Parameter.POSITIONAL_OR_KEYWORD)
+    table = {}
+    for name, par in inspect.signature(func).parameters.items():
+        if par.kind in named:
+            table[name] = None if par.default is inspect.Parameter.empty else par.default
+    if "softcap" in table:
+        table["softcap"] = 0.0
+    return table
 
 
 def get_default_args(func):
-    """utils/flash_attn_dsl.py:24-29: keyword -> default of ``func`` (or of the Python function
-    a ``torch.library`` custom op was created from), parameters without a default mapped to
-    ``None`` and ``softcap`` forced to 0.0.  The caller copies the dict before updating it."""
-    if inspect.isfunction(func):
-        return _get_default_args(func)
-    return _get_default_args(func._init_fn)
+    """Same contract as utils/flash_attn_dsl.py:14-29: keyword -> default of ``func`` (or of the Python function
+    a ``torch.library`` custom op was created from), parameters without a default mapped to ``None`` and
+    ``softcap`` forced to 0.0.  The dict is cached per function: the caller copies it before updating it, as the
+    generated code does."""
+    return _keyword_defaults(func if inspect.isfunction(func) else func._init_fn)
 
 
 def _row_strides(t: torch.Tensor):
@@ -155,18 +157,19 @@ def update_out_and_lse(out: Optional[torch.Tensor], lse: Optional[torch.Tensor],
     """utils/flash_attn_dsl.py:51-71.  First call (``out is None``) turns the block into the fp32
     accumulators; ``slice_`` merges into that sub-range of the accumulators in place; otherwise a
     functional merge."""
-    if out is None:
-        if slice_ is not None:
-            raise RuntimeError("first update_out_and_lse should not pass slice_ args")
+    first = out is None
+    if first and slice_ is not None:
+        raise RuntimeError("first update_out_and_lse should not pass slice_ args")      # the reference's message
+    if first:                                         # the block becomes the fp32 accumulators: one cast kernel
         B, Sq, Hq, D = block_out.shape
-        out = torch.empty((B, Sq, Hq, D), dtype=torch.float32, device=block_out.device)
-        lse = torch.empty((B, Sq, Hq, 1), dtype=torch.float32, device=block_out.device)
-        merge_into(None, None, block_out, block_lse, out, lse)
-    elif slice_ is not None:
-        so, sl = out[slice_], lse[slice_]
-        merge_into(so, sl, block_out, block_lse, so, sl)
-    else:
-        out, lse = _update_out_and_lse(out, lse, block_out, block_lse)
+        acc_out = torch.empty((B, Sq, Hq, D), dtype=torch.float32, device=block_out.device)
+        acc_lse = torch.empty((B, Sq, Hq, 1), dtype=torch.float32, device=block_out.device)
+        merge_into(None, None, block_out, block_lse, acc_out, acc_lse)
+        return acc_out, acc_lse
+    if slice_ is None:                                # functional: new accumulators
+        return _update_out_and_lse(out, lse, block_out, block_lse)
+    part_out, part_lse = out[slice_], lse[slice_]     # in place on the views the slice selects
+    merge_into(part_out, part_lse, block_out, block_lse, part_out, part_lse)
     return out, lse
 
 
