@@ -157,6 +157,7 @@ def other_kernels(torch, M, dev):
     dq, dkv = torch.empty_like(q), torch.empty_like(kv)
     ms = timeit(lambda: M.attn_bwd_block(do, q, kv[0], kv[1], o, lse, dq, dkv[0], dkv[1], scale))
     out["bwd_bf16_4096x4096"] = {"ms": round(ms, 4), "tflops": round(5 * unit / ms / 1e9, 1),
+                                 "pct_of_bf16_mfma_peak": round(5 * unit / ms / 1e9 / 25.0, 2),
                                  "tflops_executed": round(7 * unit / ms / 1e9, 1),
                                  "flops": "10 B H Sq Sc D algorithmic; the two-pass kernel executes 14"}
     # one rank's backward step over the same 8 chunks (dq accumulated in fp32 over the chunks, dk/dv per chunk)
