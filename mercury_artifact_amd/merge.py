@@ -286,8 +286,12 @@ def grad_accumulate(acc: Optional[torch.Tensor], block: torch.Tensor) -> torch.T
     if block.dtype != torch.bfloat16:
         raise RuntimeError("block must be bfloat16")
     block = block.contiguous()
+    if block.data_ptr() % 16:                      # a contiguous view that starts in the middle of a 16-byte group
+        block = block.clone()
     dst = torch.empty(block.shape, dtype=torch.float32, device=block.device)
     a = None if acc is None else acc.contiguous()
+    if a is not None and a.data_ptr() % 16:
+        a = a.clone()
     with torch.cuda.device(block.device):
         code = N.lib().mhip_grad_accumulate(N.ptr(a), N.ptr(block), N.ptr(dst), block.numel(), N.stream_of(block))
     N.check(code, "mhip_grad_accumulate")

@@ -153,15 +153,20 @@ def test_pack_multi_head_layout():
     assert torch.equal(M.pack_block(bo.cuda(), bl.cuda()).cpu(), O.pack_block(bo, bl))
 
 
-@pytest.mark.parametrize("n", [4096, 1001, 3])
+@pytest.mark.parametrize("n", [4096, 1001, 3, 8, 4096 * 4096 + 13, 4096 * 2048 * 5 + 8])
 def test_grad_accumulate(n):
+    """Sizes below one group of 8, with a ragged tail, and large enough for the kernel's grid-stride loop to take one
+    and two groups per pass; a block that is a view starting off a 16-byte boundary."""
     import mercury_artifact_amd as M
 
-    g = torch.Generator().manual_seed(n)
+    g = torch.Generator().manual_seed(n % 1000)
     acc = torch.randn(n, generator=g)
     blk = torch.randn(n, generator=g).bfloat16()
     assert torch.equal(M.grad_accumulate(None, blk.cuda()).cpu(), blk.float())
     assert torch.equal(M.grad_accumulate(acc.cuda(), blk.cuda()).cpu(), acc + blk.float())
+    if n > 8:
+        view = blk.cuda()[3:]
+        assert torch.equal(M.grad_accumulate(acc.cuda()[3:], view).cpu(), acc[3:] + blk[3:].float())
 
 
 @pytest.mark.parametrize("op", ["all_reduce", "reduce"])
