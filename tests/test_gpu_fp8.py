@@ -105,6 +105,33 @@ def test_fp8_block_monotone_scores(direction, binades_per_tile, causal):
     _check(out, lse, ref_a, ref_a, f"fp8 {direction} {binades_per_tile}", p_bound, check_b=False)
 
 
+@pytest.mark.parametrize("gap_nats", [4.0, 8.0])
+def test_fp8_block_with_a_dominant_first_key(gap_nats):
+    """One key of the first tile scores ``gap_nats`` above thousands of others (an attention sink).  The kernel's
+    reference stays at that key's score, so every other probability sits far down in e4m3 (at 8 nats: in its subnormal
+    range, as 2^4 P); their sum still carries a large part of the row's weight and has to come out right."""
+    import mercury_artifact_amd as M
+
+    B, Sq, Sc, H, D = 1, 256, 4096, 2, 128
+    print(f"fp8 dominant first key, gap {gap_nats}", flush=True)
+    g = torch.Generator().manual_seed(int(gap_nats))
+    q = torch.randn(B, Sq, H, D, generator=g) * 0.1
+    k = torch.randn(B, Sc, H, D, generator=g) * 0.1
+    v = torch.randn(B, Sc, H, D, generator=g)
+    scale = D ** -0.5
+    q[..., :16] = 2.0
+    k[..., :16] = 0.0
+    k[:, 0, :, :16] = gap_nats / scale / 32.0              # 16 columns x 2.0 x value = gap / scale
+    (qq, sq), (kq, sk), (vq, sv) = O.quantize_e4m3(q), O.quantize_e4m3(k), O.quantize_e4m3(v)
+    deq = (O.dequantize(qq, sq), O.dequantize(kq, sk), O.dequantize(vq, sv))
+    ref_a = O.block_attention(*deq, scale)
+    out, lse = M.attn_fwd_block(qq.cuda(), kq.cuda(), vq.cuda(), scale, q_descale=sq.cuda(), k_descale=sk.cuda(),
+                                v_descale=sv.cuda())
+    torch.cuda.synchronize()
+    p_bound = O.e4m3_p_rounding_bound(*deq, scale)
+    _check(out, lse, ref_a, ref_a, f"fp8 sink {gap_nats}", p_bound, check_b=False)
+
+
 @pytest.mark.parametrize("D,causal", [(64, False), (48, True), (16, False), (112, True)])
 def test_fp8_block_smaller_head_dims(D, causal):
     """Head dimensions below 128 (multiples of 16) through the e4m3 kernel: q, k, v and out are COLUMN slices of
